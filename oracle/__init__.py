@@ -1,0 +1,35 @@
+"""CPU oracle for the convolution / BatchNorm path -- TEST INFRASTRUCTURE ONLY.
+
+This package is a NumPy restatement of the reference's CPU algorithm
+(``src/tortto/autograd/grad_nn.py`` in samrere/pytortto 1.3.4).  It is the checker the
+GPU kernels are compared against and the CPU baseline that ``bench.py`` times; it is
+never part of the product path.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import it -- ``pytortto_amd`` must not.
+
+How each function is pinned (none of this needed an import of the reference, which
+publishes no golden vectors for this path):
+
+* ``conv2d``            brute-force nested loops, float64 evaluation, torch CPU ``F.conv2d``
+* ``conv2d_backward_x`` adjoint identity <conv(x,w),g> = <x,dgrad(g,w)> in float64,
+                        brute force, torch autograd (incl. uncovered bottom/right rows)
+* ``conv2d_backward_w`` adjoint identity <conv(x,w),g> = <w,wgrad(x,g)>, torch autograd
+* ``conv_transpose2d``  definition as dgrad of conv, torch CPU ``F.conv_transpose2d``
+                        (incl. ``output_padding``), adjointness with ``conv2d``
+* ``batch_norm_*``      closed forms (mean(y)=beta, var(y)=gamma^2 var/(var+eps)),
+                        running-stat recurrence, sum(dx)=0, sum(dx*xhat)=0,
+                        torch CPU ``F.batch_norm`` + autograd, float64 finite differences
+
+The checks live in ``tests/test_oracle_*.py``.
+"""
+from .conv import (conv2d, conv2d_backward_w, conv2d_backward_x, conv_output_size,
+                   conv_transpose_output_size, convolution_forward, convolution_backward,
+                   transposed_convolution_forward, transposed_convolution_backward)
+from .batchnorm import batch_norm_forward, batch_norm_backward
+from .nninit import conv_parameters, bn_affine_c4
+
+__all__ = [
+    'conv2d', 'conv2d_backward_w', 'conv2d_backward_x', 'conv_output_size',
+    'conv_transpose_output_size', 'convolution_forward', 'convolution_backward',
+    'transposed_convolution_forward', 'transposed_convolution_backward',
+    'batch_norm_forward', 'batch_norm_backward', 'conv_parameters', 'bn_affine_c4',
+]

@@ -1,0 +1,28 @@
+"""Shared convolution parameter grids for the oracle and GPU parity tests."""
+
+# (N, C, H, W, K, R, S, stride, padding, dilation, groups)
+CONV_CASES = [
+    (2, 4, 8, 8, 6, 3, 3, (1, 1), (1, 1), (1, 1), 1),
+    (2, 4, 8, 8, 6, 3, 3, (2, 2), (1, 1), (1, 1), 1),     # (H+2p-d(R-1)-1) % s != 0: uncovered rows
+    (2, 4, 9, 7, 6, 3, 2, (2, 1), (0, 1), (1, 2), 2),
+    (1, 6, 10, 11, 4, 2, 3, (3, 2), (2, 0), (2, 1), 2),
+    (3, 3, 7, 7, 5, 1, 1, (1, 1), (0, 0), (1, 1), 1),     # 1x1: plain matrix product
+    (2, 4, 8, 8, 8, 1, 1, (2, 2), (0, 0), (1, 1), 1),     # 1x1 stride 2 (shortcut): 3/4 of dx is zero
+    (2, 3, 12, 12, 4, 7, 7, (2, 2), (3, 3), (1, 1), 1),   # stem-like
+    (2, 8, 6, 5, 8, 3, 3, (1, 1), (2, 2), (2, 2), 4),
+    (1, 2, 5, 5, 2, 5, 5, (1, 1), (0, 0), (1, 1), 1),     # kernel == input
+    (2, 4, 8, 8, 4, 4, 4, (2, 2), (1, 1), (1, 1), 1),     # DCGAN-style geometry, as a conv
+    (2, 6, 9, 9, 3, 3, 3, (3, 3), (1, 1), (1, 1), 3),     # stride 3 with dead input rows
+    (2, 4, 11, 10, 6, 3, 3, (2, 3), (1, 2), (2, 1), 1),   # gcd(stride, dilation) > 1 in H
+]
+
+# (N, C_in, H, W, C_out, R, S, stride, padding, output_padding, dilation, groups)
+CONVT_CASES = [
+    (2, 5, 1, 1, 6, 4, 4, (1, 1), (0, 0), (0, 0), (1, 1), 1),   # DCGAN first layer geometry
+    (2, 6, 4, 4, 4, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),   # DCGAN upsampling geometry
+    (2, 4, 5, 6, 6, 3, 3, (2, 2), (1, 1), (1, 1), (1, 1), 2),
+    (1, 4, 5, 4, 2, 3, 2, (3, 2), (1, 0), (2, 1), (2, 1), 2),
+    (2, 3, 6, 6, 5, 1, 1, (1, 1), (0, 0), (0, 0), (1, 1), 1),
+    (2, 4, 4, 5, 4, 3, 3, (2, 2), (0, 0), (1, 0), (2, 2), 1),   # gcd(stride, dilation) = 2
+    (1, 2, 3, 3, 2, 2, 2, (3, 3), (0, 0), (2, 2), (1, 1), 1),   # stride > kernel: holes in the output
+]
