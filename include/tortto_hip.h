@@ -1,0 +1,132 @@
+/*
+ * libtortto_hip.so -- C ABI of the MI355X (gfx950) convolution / BatchNorm path for tortto.
+ *
+ * The reference (samrere/pytortto 1.3.4) is pure Python: its GPU backend is "the same NumPy
+ * expression executed by CuPy".  The functions below are what a native backend for that path
+ * binds instead; each one names the reference call site it replaces
+ * (paths relative to the reference's src/tortto/).
+ *
+ * Conventions
+ *   - every function returns 0 on success, non-zero on failure; tt_last_error() then holds a
+ *     message.  Nothing throws or aborts across this boundary.
+ *   - all tensor pointers are DEVICE pointers to C-contiguous float32 NCHW data unless a
+ *     parameter is documented as a host pointer.  Outputs are caller-allocated.
+ *   - kernels are enqueued on one library-owned HIP stream and return immediately;
+ *     tt_sync() / tt_memcpy_d2h() wait for them.  One caller thread at a time.
+ *   - tensors are limited to 2^31-1 elements each (32-bit element offsets in the kernels);
+ *     larger ones are rejected with an error.
+ */
+#ifndef TORTTO_HIP_H
+#define TORTTO_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- runtime: device, memory, stream (replaces cupy.ndarray allocation, cparray(x) H2D and
+ *      x.get() D2H at autograd/grad_fcn.py:859-865, :873-877; nn/modules/module.py:108-122) ---- */
+
+const char* tt_last_error(void);
+int tt_init(int device);
+/* name: host buffer of name_len bytes; the other outputs are host pointers and may be NULL. */
+int tt_device_info(char* name, int name_len, int* compute_units, int* clock_khz,
+                   int* lds_bytes_per_block, size_t* total_mem_bytes);
+int tt_malloc(void** ptr, size_t bytes);      /* pooled: freed blocks are reused by size class */
+int tt_free(void* ptr);
+int tt_empty_cache(void);                     /* return pooled blocks and the workspace to HIP */
+int tt_mem_stats(size_t* bytes_in_use, size_t* bytes_pooled, size_t* workspace_bytes);
+int tt_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes);   /* synchronous */
+int tt_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes);   /* synchronous */
+int tt_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes);    /* stream-ordered */
+int tt_memset(void* dst_dev, int byte_value, size_t bytes);             /* stream-ordered */
+int tt_sync(void);
+
+/* HIP events on the library stream, for timing kernels from the host side. */
+int tt_event_create(void** event);
+int tt_event_record(void* event);
+int tt_event_elapsed_ms(void* start, void* stop, float* ms);   /* waits for `stop` */
+int tt_event_destroy(void* event);
+
+/* ---- convolution ------------------------------------------------------------------------- */
+
+/* y[N,K,P,Q] = conv(x[N,C,H,W], w[K,C/groups,R,S]) (+ bias[K] if not NULL).
+ * Replaces _padding + _sliding_window_view + einsum and the bias add:
+ * autograd/grad_nn.py:595-643 (called from :709-711).
+ * P = floor((H + 2*ph - dh*(R-1) - 1)/sh) + 1, likewise Q (grad_nn.py:565-566). */
+int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* y,
+                      int N, int C, int H, int W, int K, int R, int S,
+                      int sh, int sw, int ph, int pw, int dh, int dw, int groups);
+
+/* dx[N,C,Hx,Wx] = sum over k,r,s of dy[N,K,P,Q] * w[K,C/groups,R,S] (+ bias[C] if not NULL):
+ * the input gradient of the convolution above, and -- with x as `dy`, the [C_in,C_out/g,R,S]
+ * transposed-convolution weight as `w`, K = C_in, C = C_out -- the forward pass of
+ * ConvTranspose2d.  Hx, Wx are explicit so that output_padding and rows the forward pass
+ * never covered (zero-filled) are handled.  Replaces _dilate + flip + _padding + einsum + crop
+ * + pad: autograd/grad_nn.py:659-682 (called from :733 and :755-757). */
+int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx,
+                        int N, int C, int Hx, int Wx, int K, int R, int S,
+                        int sh, int sw, int ph, int pw, int dh, int dw, int groups,
+                        int P, int Q);
+
+/* dw[K,C/groups,R,S] = sum over n,p,q of x~[n,c,p*sh+r*dh-ph,q*sw+s*dw-pw] * dy[n,k,p,q]
+ * (x~ = x zero-padded).  Deterministic: fixed split of the reduction, partial sums combined
+ * in float64.  Replaces _conv2d_backward_w: autograd/grad_nn.py:646-656 (called from :731
+ * and, with the roles of x and dy exchanged by the caller, :776). */
+int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw,
+                        int N, int C, int H, int W, int K, int R, int S,
+                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups,
+                        int P, int Q);
+
+/* out[K] = sum over n and the HW plane of t[N,K,HW]: the bias gradient gd0.sum((0,2,3)),
+ * autograd/grad_nn.py:728, :774. */
+int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW);
+
+/* ---- BatchNorm (x viewed as [N, C, HW]) ---------------------------------------------------- */
+
+/* Training forward, autograd/grad_nn.py:921-930 and :942-959:
+ *   mean/var(biased) over (n,hw); save_mean[C], save_var_eps[C] = var+eps, save_sd[C] = sqrt(var+eps);
+ *   y = (x-mean)/sd*gamma+beta (gamma, beta may be NULL);
+ *   if running_mean_in/var_in are not NULL:
+ *     running_mean_out = (1-momentum)*running_mean_in + momentum*mean
+ *     running_var_out  = (1-momentum)*running_var_in  + momentum*var*(M/(M-1)),  M = N*HW
+ *   (in/out may alias).  Returns an error when M == 1 (grad_nn.py:899-904). */
+int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y,
+                        float* save_mean, float* save_var_eps, float* save_sd,
+                        const float* running_mean_in, const float* running_var_in,
+                        float* running_mean_out, float* running_var_out,
+                        double momentum, double eps, int N, int C, int HW);
+
+/* Normalisation with given statistics (eval mode), autograd/grad_nn.py:931-959:
+ * save_* are written from mean[C]/var[C] exactly as in training so that backward can follow. */
+int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, float* y,
+                       const float* mean, const float* var,
+                       float* save_mean, float* save_var_eps, float* save_sd,
+                       double eps, int N, int C, int HW);
+
+/* Backward, autograd/grad_nn.py:966-989.  dx, dgamma, dbeta may each be NULL (not needed):
+ *   dbeta = sum dy; dgamma = sum dy*(x-mean)/sd;
+ *   dx = ((M*g - sum g) - (x-mean)/var_eps * sum(g*(x-mean))) / M / sd,  g = dy*gamma. */
+int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
+                  const float* save_mean, const float* save_var_eps, const float* save_sd,
+                  float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
+
+/* ---- elementwise glue so whole stacks stay on the device ----------------------------------- */
+
+/* y = max(x, 0) (autograd/grad_nn.py:33-69); dx = dy * (y > 0). */
+int tt_relu_fwd_f32(const float* x, float* y, size_t n);
+int tt_relu_bwd_f32(const float* dy, const float* y, float* dx, size_t n);
+/* out = a + b (residual Add, autograd/grad_fcn.py:177-203). */
+int tt_add_f32(const float* a, const float* b, float* out, size_t n);
+/* acc += alpha * v: gradient accumulation `fn.grad[ind] += grad` (tensor.py:596-599,
+ * autograd/function.py:88-93). */
+int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n);
+/* dst[i] = value */
+int tt_fill_f32(float* dst, float value, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORTTO_HIP_H */

@@ -1,0 +1,132 @@
+"""ctypes binding of ``libtortto_hip.so`` -- the only door from Python to the GPU.
+
+The prototypes below restate ``include/tortto_hip.h``.  The library is loaded on first use
+(``lib()``); if it has not been built, or no MI355X is visible, that raises -- there is no
+CPU fallback behind this module.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
+
+from .build import LIB_PATH
+
+_P = c_void_p
+_I = c_int
+
+# name -> argument types (every function returns int, except tt_last_error)
+PROTOTYPES = {
+    'tt_init': [_I],
+    'tt_device_info': [c_char_p, _I, POINTER(c_int), POINTER(c_int), POINTER(c_int), POINTER(c_size_t)],
+    'tt_malloc': [POINTER(c_void_p), c_size_t],
+    'tt_free': [_P],
+    'tt_empty_cache': [],
+    'tt_mem_stats': [POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)],
+    'tt_memcpy_h2d': [_P, _P, c_size_t],
+    'tt_memcpy_d2h': [_P, _P, c_size_t],
+    'tt_memcpy_d2d': [_P, _P, c_size_t],
+    'tt_memset': [_P, _I, c_size_t],
+    'tt_sync': [],
+    'tt_event_create': [POINTER(c_void_p)],
+    'tt_event_record': [_P],
+    'tt_event_elapsed_ms': [_P, _P, POINTER(c_float)],
+    'tt_event_destroy': [_P],
+    'tt_conv2d_fwd_f32': [_P, _P, _P, _P] + [_I] * 14,
+    'tt_conv2d_dgrad_f32': [_P, _P, _P, _P] + [_I] * 16,
+    'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
+    'tt_channel_sum_f32': [_P, _P, _I, _I, _I],
+    'tt_bn_fwd_train_f32': [_P] * 11 + [c_double, c_double, _I, _I, _I],
+    'tt_bn_fwd_eval_f32': [_P] * 9 + [c_double, _I, _I, _I],
+    'tt_bn_bwd_f32': [_P] * 9 + [_I, _I, _I],
+    'tt_relu_fwd_f32': [_P, _P, c_size_t],
+    'tt_relu_bwd_f32': [_P, _P, _P, c_size_t],
+    'tt_add_f32': [_P, _P, _P, c_size_t],
+    'tt_axpy_f32': [c_float, _P, _P, c_size_t],
+    'tt_fill_f32': [_P, c_float, c_size_t],
+}
+
+_lib = None
+_ready = False
+
+
+def load_library(path=None):
+    """dlopen the library and attach prototypes (no GPU call is made)."""
+    global _lib
+    if _lib is None:
+        path = path or LIB_PATH
+        if not os.path.exists(path):
+            raise RuntimeError(f'{path} has not been built: run `python -m pytortto_amd.build` '
+                               f'(there is no CPU fallback for the device path)')
+        handle = ctypes.CDLL(path)
+        handle.tt_last_error.restype = c_char_p
+        handle.tt_last_error.argtypes = []
+        for name, args in PROTOTYPES.items():
+            fn = getattr(handle, name)
+            fn.restype = c_int
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise RuntimeError(_lib.tt_last_error().decode(errors='replace'))
+
+
+def lib():
+    """The loaded library with ``tt_init(0)`` done."""
+    global _ready
+    handle = load_library()
+    if not _ready:
+        check(handle.tt_init(0))
+        _ready = True
+    return handle
+
+
+def call(name, *args):
+    """Call ``name`` through the C ABI and raise ``RuntimeError(tt_last_error())`` on failure."""
+    check(getattr(lib(), name)(*args))
+
+
+def is_available():
+    """True when the library is built and a gfx950 device answers."""
+    try:
+        lib()
+        return True
+    except (RuntimeError, OSError):
+        return False
+
+
+def device_info():
+    name = ctypes.create_string_buffer(256)
+    cus, khz, lds, mem = c_int(), c_int(), c_int(), c_size_t()
+    call('tt_device_info', name, 256, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(lds), ctypes.byref(mem))
+    return {'name': name.value.decode(), 'compute_units': cus.value, 'clock_khz': khz.value,
+            'lds_bytes_per_block': lds.value, 'total_mem_bytes': mem.value}
+
+
+def synchronize():
+    call('tt_sync')
+
+
+class Event:
+    """HIP event on the library stream."""
+
+    def __init__(self):
+        self._h = c_void_p()
+        call('tt_event_create', ctypes.byref(self._h))
+
+    def record(self):
+        call('tt_event_record', self._h)
+        return self
+
+    def elapsed_ms(self, later):
+        ms = c_float()
+        call('tt_event_elapsed_ms', self._h, later._h, ctypes.byref(ms))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.tt_event_destroy(self._h)
+        except Exception:
+            pass

@@ -1,0 +1,543 @@
+// BatchNorm2d training forward/backward for NCHW float32 on gfx950 -- HBM-bound kernels.
+//
+// x is viewed as [N, C, HW]: channel c owns N planes of HW contiguous floats, C*HW apart.
+// Forward  = sweep 1 (read x: per-channel shifted moments)  + sweep 2 (read x, write y).
+// Backward = sweep 1 (read x, dy: sum dy, sum dy*(x-mean))  + sweep 2 (read x, dy, write dx).
+// Algorithmic traffic: 3*S forward, 5*S backward, S = 4*N*C*HW bytes.
+//
+// Grid is (splits, C): one block column per channel, `splits` blocks share a channel's planes
+// so that even C = 64 fills 256 CUs.  Each block leaves an fp64 partial; the second sweep's
+// blocks each re-reduce their channel's <= 64 partials in their prologue (cheaper than a
+// separate finalize launch), and the block with split 0 writes the per-channel outputs.
+// The second sweep walks channels, splits and planes in the opposite order of the first one,
+// so what the first sweep touched last -- still resident in the memory-side cache -- is read
+// first.
+//
+// Numerics: moments are taken about shift = x[0,c,0,0] (a sample of the channel, so within a
+// few sigma of its mean): float32 accumulation inside one plane per lane, float64 across
+// planes, lanes, waves and blocks; var = E[d^2] - E[d]^2 in float64.  This keeps the
+// cancellation that a raw one-pass E[x^2]-E[x]^2 suffers for inputs with |mean| >> sigma away.
+#include "tt_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / tt::kWave;
+constexpr int kMaxSplits = 64;
+
+// ---- wave64 all-reduce (sum) with DPP + ds_swizzle ------------------------------------------
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, false));
+}
+template <int kCtrl>
+__device__ __forceinline__ double dpp_d(double v) {
+  int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), kCtrl, 0xf, 0xf, false);
+  int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), kCtrl, 0xf, 0xf, false);
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double swz16_d(double v) {  // lane ^ 16 inside each 32-lane half
+  int lo = __builtin_amdgcn_ds_swizzle(__double2loint(v), 0x401f);
+  int hi = __builtin_amdgcn_ds_swizzle(__double2hiint(v), 0x401f);
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double readlane_d(double v, int lane) {
+  int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
+  int hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+  return __hiloint2double(hi, lo);
+}
+
+// Sum over the 64 lanes of a wave; every lane gets the (wave-uniform) result.
+__device__ __forceinline__ double wave_sum(double v) {
+  v += dpp_d<0xB1>(v);   // quad_perm [1,0,3,2]   : lane ^ 1
+  v += dpp_d<0x4E>(v);   // quad_perm [2,3,0,1]   : lane ^ 2
+  v += dpp_d<0x141>(v);  // row_half_mirror       : joins the two quads of each 8
+  v += dpp_d<0x140>(v);  // row_mirror            : joins the two 8s of each row of 16
+  v += swz16_d(v);       // joins the two rows of each 32-lane half
+  return readlane_d(v, 0) + readlane_d(v, 32);
+}
+
+// Two sums per block: wave_sum, then the four waves through LDS.  Result valid in all threads.
+__device__ __forceinline__ void block_sum2(double& a, double& b, double* lds /* 2*kWaves */) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    lds[2 * wave] = a;
+    lds[2 * wave + 1] = b;
+  }
+  __syncthreads();
+  a = 0;
+  b = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    a += lds[2 * w];
+    b += lds[2 * w + 1];
+  }
+  __syncthreads();
+}
+
+// Re-reduce one channel's partials (<= 64, one per lane) -- wave-uniform result.
+__device__ __forceinline__ void load_partials(const double2* __restrict__ partial, int c, int splits,
+                                              double& a, double& b) {
+  const int lane = threadIdx.x & 63;
+  double2 p = make_double2(0.0, 0.0);
+  if (lane < splits) p = partial[(size_t)c * splits + lane];
+  a = wave_sum(p.x);
+  b = wave_sum(p.y);
+}
+
+struct Geometry {
+  int N, C, HW;         // HW in floats
+  int splits;           // gridDim.x
+  int per_block;        // planes (plane kernels) or vectors (flat kernels) per block
+  tt::FastDiv hwv_div;  // flat kernels: divisor HW / VEC
+};
+
+// ---- sweep 1: partial sums ---------------------------------------------------------------------
+// kKind 0: a = sum (x - shift),  b = sum (x - shift)^2         (shift = x[0,c,0,0])
+// kKind 1: a = sum dy,           b = sum dy * (x - mean[c])
+// kKind 2: a = sum x,            b unused                        (bias gradient)
+
+// Plane kernel: HW % 4 == 0 and HW/4 >= 32.  Each wave streams whole planes with float4 loads.
+template <int kKind>
+__global__ __launch_bounds__(kThreads) void bn_reduce_planes(const float* __restrict__ x,
+                                                             const float* __restrict__ dy,
+                                                             const float* __restrict__ mean,
+                                                             double2* __restrict__ partial, Geometry g) {
+  __shared__ double lds[2 * kWaves];
+  const int c = blockIdx.y, split = blockIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  constexpr bool kBwd = kKind == 1;
+  const int hw4 = g.HW >> 2;
+  const float ref = kKind == 1 ? mean[c] : (kKind == 0 ? x[(size_t)c * g.HW] : 0.f);
+  const int n0 = split * g.per_block;
+  const int n1 = min(g.N, n0 + g.per_block);
+  double sa = 0.0, sb = 0.0;
+  for (int n = n0 + wave; n < n1; n += kWaves) {
+    const size_t off = ((size_t)n * g.C + c) * g.HW;
+    const float4* __restrict__ px = reinterpret_cast<const float4*>(x + off);
+    const float4* __restrict__ pg = reinterpret_cast<const float4*>(dy + (kBwd ? off : 0));
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+#pragma unroll 4
+    for (int i = lane; i < hw4; i += tt::kWave) {
+      float4 v = px[i];
+      v.x -= ref; v.y -= ref; v.z -= ref; v.w -= ref;
+      if (kBwd) {
+        const float4 gq = pg[i];
+        a.x += gq.x; a.y += gq.y; a.z += gq.z; a.w += gq.w;
+        b.x = fmaf(gq.x, v.x, b.x); b.y = fmaf(gq.y, v.y, b.y);
+        b.z = fmaf(gq.z, v.z, b.z); b.w = fmaf(gq.w, v.w, b.w);
+      } else {
+        a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+        if (kKind == 0) {
+          b.x = fmaf(v.x, v.x, b.x); b.y = fmaf(v.y, v.y, b.y);
+          b.z = fmaf(v.z, v.z, b.z); b.w = fmaf(v.w, v.w, b.w);
+        }
+      }
+    }
+    sa += ((double)a.x + (double)a.y) + ((double)a.z + (double)a.w);
+    sb += ((double)b.x + (double)b.y) + ((double)b.z + (double)b.w);
+  }
+  block_sum2(sa, sb, lds);
+  if (threadIdx.x == 0) partial[(size_t)c * g.splits + split] = make_double2(sa, sb);
+}
+
+// Flat kernel: any HW.  Vector index e over the channel's N*HW/VEC vectors, n = e / (HW/VEC).
+template <int kKind, int VEC>
+__global__ __launch_bounds__(kThreads) void bn_reduce_flat(const float* __restrict__ x,
+                                                           const float* __restrict__ dy,
+                                                           const float* __restrict__ mean,
+                                                           double2* __restrict__ partial, Geometry g) {
+  __shared__ double lds[2 * kWaves];
+  const int c = blockIdx.y, split = blockIdx.x;
+  const uint32_t hwv = (uint32_t)g.HW / VEC;
+  constexpr bool kBwd = kKind == 1;
+  const uint32_t total = (uint32_t)g.N * hwv;
+  const float ref = kKind == 1 ? mean[c] : (kKind == 0 ? x[(size_t)c * g.HW] : 0.f);
+  const uint32_t e0 = (uint32_t)split * (uint32_t)g.per_block;
+  const uint32_t e1 = min(total, e0 + (uint32_t)g.per_block);
+  double sa = 0.0, sb = 0.0;
+  for (uint32_t e = e0 + threadIdx.x; e < e1; e += kThreads) {
+    const uint32_t n = tt::fd_div(e, g.hwv_div);
+    const uint32_t r = e - n * hwv;
+    const size_t off = ((size_t)n * g.C + c) * g.HW + (size_t)r * VEC;
+    float v[VEC], gq[VEC] = {};
+    if constexpr (VEC == 4) {
+      const float4 t = *reinterpret_cast<const float4*>(x + off);
+      v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+      if constexpr (kBwd) {
+        const float4 u = *reinterpret_cast<const float4*>(dy + off);
+        gq[0] = u.x; gq[1] = u.y; gq[2] = u.z; gq[3] = u.w;
+      }
+    } else {
+      v[0] = x[off];
+      if constexpr (kBwd) gq[0] = dy[off];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = v[j] - ref;
+      if (kBwd) {
+        sa += (double)gq[j];
+        sb += (double)gq[j] * (double)d;
+      } else {
+        sa += (double)d;
+        if (kKind == 0) sb += (double)d * (double)d;
+      }
+    }
+  }
+  block_sum2(sa, sb, lds);
+  if (threadIdx.x == 0) partial[(size_t)c * g.splits + split] = make_double2(sa, sb);
+}
+
+// ---- sweep 2: y = (x - m) * k1 + k0      (forward)
+//               dx = dy * k1 + (x - m) * k2 + k0   (backward)
+struct Coef {
+  float m, k0, k1, k2;
+};
+
+template <bool kBwd>
+__device__ __forceinline__ float4 apply4(const float4 v, const float4 gq, const Coef k) {
+  float4 o;
+  if (kBwd) {
+    o.x = fmaf(gq.x, k.k1, fmaf(v.x - k.m, k.k2, k.k0));
+    o.y = fmaf(gq.y, k.k1, fmaf(v.y - k.m, k.k2, k.k0));
+    o.z = fmaf(gq.z, k.k1, fmaf(v.z - k.m, k.k2, k.k0));
+    o.w = fmaf(gq.w, k.k1, fmaf(v.w - k.m, k.k2, k.k0));
+  } else {
+    o.x = fmaf(v.x - k.m, k.k1, k.k0);
+    o.y = fmaf(v.y - k.m, k.k1, k.k0);
+    o.z = fmaf(v.z - k.m, k.k1, k.k0);
+    o.w = fmaf(v.w - k.m, k.k1, k.k0);
+  }
+  return o;
+}
+
+template <bool kBwd>
+__device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const float* __restrict__ dy,
+                                              float* __restrict__ out, const Geometry& g, int c, int split,
+                                              const Coef k) {
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int hw4 = g.HW >> 2;
+  const int n0 = split * g.per_block;
+  const int n1 = min(g.N, n0 + g.per_block);
+  for (int n = n1 - 1 - wave; n >= n0; n -= kWaves) {
+    const size_t off = ((size_t)n * g.C + c) * g.HW;
+    const float4* __restrict__ px = reinterpret_cast<const float4*>(x + off);
+    const float4* __restrict__ pg = reinterpret_cast<const float4*>(dy + (kBwd ? off : 0));
+    float4* __restrict__ po = reinterpret_cast<float4*>(out + off);
+#pragma unroll 4
+    for (int i = lane; i < hw4; i += tt::kWave) {
+      const float4 v = px[i];
+      float4 gq = v;
+      if (kBwd) gq = pg[i];
+      po[i] = apply4<kBwd>(v, gq, k);
+    }
+  }
+}
+
+template <bool kBwd, int VEC>
+__device__ __forceinline__ void sweep2_flat(const float* __restrict__ x, const float* __restrict__ dy,
+                                            float* __restrict__ out, const Geometry& g, int c, int split,
+                                            const Coef k) {
+  const uint32_t hwv = (uint32_t)g.HW / VEC;
+  const uint32_t total = (uint32_t)g.N * hwv;
+  const uint32_t e0 = (uint32_t)split * (uint32_t)g.per_block;
+  const uint32_t e1 = min(total, e0 + (uint32_t)g.per_block);
+  for (uint32_t e = e0 + threadIdx.x; e < e1; e += kThreads) {
+    const uint32_t n = tt::fd_div(e, g.hwv_div);
+    const uint32_t r = e - n * hwv;
+    const size_t off = ((size_t)n * g.C + c) * g.HW + (size_t)r * VEC;
+    if constexpr (VEC == 4) {
+      const float4 v = *reinterpret_cast<const float4*>(x + off);
+      float4 gq = v;
+      if (kBwd) gq = *reinterpret_cast<const float4*>(dy + off);
+      *reinterpret_cast<float4*>(out + off) = apply4<kBwd>(v, gq, k);
+    } else {
+      const float v = x[off];
+      if (kBwd)
+        out[off] = fmaf(dy[off], k.k1, fmaf(v - k.m, k.k2, k.k0));
+      else
+        out[off] = fmaf(v - k.m, k.k1, k.k0);
+    }
+  }
+}
+
+struct FwdArgs {
+  const float* x;
+  const float* gamma;
+  const float* beta;
+  float* y;
+  float* save_mean;
+  float* save_var_eps;
+  float* save_sd;
+  const float* rm_in;
+  const float* rv_in;
+  float* rm_out;
+  float* rv_out;
+  const float* given_mean;  // eval mode: statistics are inputs, no partials
+  const float* given_var;
+  const double2* partial;
+  float one_minus_mom, mom, unbias, eps;
+};
+
+// kMode: 0 planes, 1 flat VEC=4, 2 flat VEC=1
+template <int kMode>
+__global__ __launch_bounds__(kThreads) void bn_fwd_apply(FwdArgs a, Geometry g) {
+  __shared__ Coef sk;
+  const int c = g.C - 1 - (int)blockIdx.y;
+  const int split = g.splits - 1 - (int)blockIdx.x;
+  if (threadIdx.x < tt::kWave) {
+    float mean, var;
+    if (a.given_mean) {
+      mean = a.given_mean[c];
+      var = a.given_var[c];
+    } else {
+      double s1, s2;
+      load_partials(a.partial, c, g.splits, s1, s2);
+      const double m = (double)g.N * (double)g.HW;
+      const double shift = (double)a.x[(size_t)c * g.HW];
+      const double d1 = s1 / m;
+      mean = (float)(shift + d1);
+      var = (float)fmax(s2 / m - d1 * d1, 0.0);
+    }
+    const float var_eps = __fadd_rn(var, a.eps);
+    const float sd = __fsqrt_rn(var_eps);
+    const float gam = a.gamma ? a.gamma[c] : 1.0f;
+    const float bet = a.beta ? a.beta[c] : 0.0f;
+    if (threadIdx.x == 0) {
+      sk.m = mean;
+      sk.k1 = __fdiv_rn(gam, sd);
+      sk.k0 = bet;
+      sk.k2 = 0.f;
+      if (split == 0) {
+        a.save_mean[c] = mean;
+        a.save_var_eps[c] = var_eps;
+        a.save_sd[c] = sd;
+        if (a.rm_in && !a.given_mean) {
+          // separate roundings, as NumPy evaluates (1-m)*rm + m*mean on float32 arrays
+          a.rm_out[c] = __fadd_rn(__fmul_rn(a.one_minus_mom, a.rm_in[c]), __fmul_rn(a.mom, mean));
+          a.rv_out[c] =
+              __fadd_rn(__fmul_rn(a.one_minus_mom, a.rv_in[c]), __fmul_rn(a.mom, __fmul_rn(var, a.unbias)));
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const Coef k = sk;
+  if (kMode == 0) sweep2_planes<false>(a.x, a.x, a.y, g, c, split, k);
+  if (kMode == 1) sweep2_flat<false, 4>(a.x, a.x, a.y, g, c, split, k);
+  if (kMode == 2) sweep2_flat<false, 1>(a.x, a.x, a.y, g, c, split, k);
+}
+
+struct BwdArgs {
+  const float* x;
+  const float* dy;
+  const float* gamma;
+  const float* save_mean;
+  const float* save_var_eps;
+  const float* save_sd;
+  float* dx;
+  float* dgamma;
+  float* dbeta;
+  const double2* partial;
+};
+
+template <int kMode>
+__global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) {
+  __shared__ Coef sk;
+  const int c = g.C - 1 - (int)blockIdx.y;
+  const int split = g.splits - 1 - (int)blockIdx.x;
+  if (threadIdx.x < tt::kWave) {
+    double s_dy, s_dyxmu;
+    load_partials(a.partial, c, g.splits, s_dy, s_dyxmu);
+    if (threadIdx.x == 0) {
+      const double m = (double)g.N * (double)g.HW;
+      const double sd = (double)a.save_sd[c];
+      const double var_eps = (double)a.save_var_eps[c];
+      const double k1 = (a.gamma ? (double)a.gamma[c] : 1.0) / sd;
+      sk.m = a.save_mean[c];
+      sk.k1 = (float)k1;
+      sk.k0 = (float)(-k1 * s_dy / m);
+      sk.k2 = (float)(-k1 * s_dyxmu / (m * var_eps));
+      if (split == 0) {
+        if (a.dbeta) a.dbeta[c] = (float)s_dy;
+        if (a.dgamma) a.dgamma[c] = (float)(s_dyxmu / sd);
+      }
+    }
+  }
+  if (a.dx == nullptr) return;
+  __syncthreads();
+  const Coef k = sk;
+  if (kMode == 0) sweep2_planes<true>(a.x, a.dy, a.dx, g, c, split, k);
+  if (kMode == 1) sweep2_flat<true, 4>(a.x, a.dy, a.dx, g, c, split, k);
+  if (kMode == 2) sweep2_flat<true, 1>(a.x, a.dy, a.dx, g, c, split, k);
+}
+
+// ---- host side -------------------------------------------------------------------------------------
+
+int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// Picks the kernel flavour and how a channel is shared between blocks.
+int plan(int N, int C, int HW, Geometry* g, int* mode) {
+  g->N = N;
+  g->C = C;
+  g->HW = HW;
+  const int target_blocks = 4096;  // ~2 resident rounds of 8 blocks on each of 256 CUs
+  int want = target_blocks / C;
+  if (want < 1) want = 1;
+  if (want > kMaxSplits) want = kMaxSplits;
+  if (HW % 4 == 0 && HW / 4 >= 32) {
+    *mode = 0;
+    int ppb = ceil_div(N, want);
+    ppb = (ppb + kWaves - 1) / kWaves * kWaves;  // whole rounds of one plane per wave
+    g->per_block = ppb;
+    g->splits = ceil_div(N, ppb);
+    g->hwv_div = tt::make_fastdiv(1);
+  } else {
+    const int vec = (HW % 4 == 0) ? 4 : 1;
+    *mode = vec == 4 ? 1 : 2;
+    const long long vectors = (long long)N * (HW / vec);
+    long long per = (vectors + want - 1) / want;
+    per = (per + kThreads - 1) / kThreads * kThreads;
+    g->per_block = (int)per;
+    g->splits = ceil_div(vectors, per);
+    g->hwv_div = tt::make_fastdiv((uint32_t)(HW / vec));
+  }
+  return 0;
+}
+
+int check_shape(const char* fn, int N, int C, int HW) {
+  TT_REQUIRE(N > 0 && C > 0 && HW > 0, "%s: N, C, HW must be positive (got %d, %d, %d)", fn, N, C, HW);
+  TT_REQUIRE(tt::fits_i32((long long)N * C * HW), "%s: tensor of %lld elements exceeds 2^31-1", fn,
+             (long long)N * C * HW);
+  TT_REQUIRE(C <= 65535, "%s: more than 65535 channels are not supported", fn);
+  return 0;
+}
+
+template <int kKind>
+void launch_reduce(int mode, dim3 grid, const float* x, const float* dy, const float* mean, double2* partial,
+                   const Geometry& g) {
+  hipStream_t st = tt::stream();
+  if (mode == 0) bn_reduce_planes<kKind><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
+  if (mode == 1) bn_reduce_flat<kKind, 4><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
+  if (mode == 2) bn_reduce_flat<kKind, 1><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
+}
+
+// out[c] = sum of channel c's partials (bias gradient).
+__global__ __launch_bounds__(tt::kWave) void channel_sum_finish(const double2* __restrict__ partial,
+                                                               float* __restrict__ out, int splits) {
+  double a, b;
+  load_partials(partial, blockIdx.x, splits, a, b);
+  if (threadIdx.x == 0) out[blockIdx.x] = (float)a;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
+                        float* save_var_eps, float* save_sd, const float* running_mean_in,
+                        const float* running_var_in, float* running_mean_out, float* running_var_out,
+                        double momentum, double eps, int N, int C, int HW) {
+  TT_REQUIRE_INIT();
+  if (check_shape("tt_bn_fwd_train_f32", N, C, HW)) return -1;
+  TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "tt_bn_fwd_train_f32: null tensor pointer");
+  const long long m = (long long)N * HW;
+  TT_REQUIRE(m > 1, "Expected more than 1 value per channel when training, got input size [%d, %d, %d]", N, C, HW);
+  const bool track = running_mean_in && running_var_in;
+  TT_REQUIRE(!track || (running_mean_out && running_var_out),
+             "tt_bn_fwd_train_f32: running statistics given without output buffers");
+  Geometry g;
+  int mode;
+  plan(N, C, HW, &g, &mode);
+  void* ws;
+  if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
+  dim3 grid(g.splits, C);
+  launch_reduce<0>(mode, grid, x, x, nullptr, (double2*)ws, g);
+  TT_LAUNCH_CHECK();
+  FwdArgs a{};
+  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
+  a.save_mean = save_mean; a.save_var_eps = save_var_eps; a.save_sd = save_sd;
+  a.rm_in = track ? running_mean_in : nullptr; a.rv_in = track ? running_var_in : nullptr;
+  a.rm_out = running_mean_out; a.rv_out = running_var_out;
+  a.given_mean = nullptr; a.given_var = nullptr;
+  a.partial = (const double2*)ws;
+  a.one_minus_mom = (float)(1.0 - momentum);
+  a.mom = (float)momentum;
+  a.unbias = (float)((double)m / (double)(m - 1));
+  a.eps = (float)eps;
+  hipStream_t st = tt::stream();
+  if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, float* y, const float* mean,
+                       const float* var, float* save_mean, float* save_var_eps, float* save_sd, double eps, int N,
+                       int C, int HW) {
+  TT_REQUIRE_INIT();
+  if (check_shape("tt_bn_fwd_eval_f32", N, C, HW)) return -1;
+  TT_REQUIRE(x && y && mean && var && save_mean && save_var_eps && save_sd,
+             "tt_bn_fwd_eval_f32: null tensor pointer");
+  Geometry g;
+  int mode;
+  plan(N, C, HW, &g, &mode);
+  dim3 grid(g.splits, C);
+  FwdArgs a{};
+  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
+  a.save_mean = save_mean; a.save_var_eps = save_var_eps; a.save_sd = save_sd;
+  a.given_mean = mean; a.given_var = var;
+  a.eps = (float)eps;
+  hipStream_t st = tt::stream();
+  if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                  const float* save_var_eps, const float* save_sd, float* dx, float* dgamma, float* dbeta, int N,
+                  int C, int HW) {
+  TT_REQUIRE_INIT();
+  if (check_shape("tt_bn_bwd_f32", N, C, HW)) return -1;
+  TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "tt_bn_bwd_f32: null tensor pointer");
+  if (!dx && !dgamma && !dbeta) return 0;
+  Geometry g;
+  int mode;
+  plan(N, C, HW, &g, &mode);
+  void* ws;
+  if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
+  dim3 grid(g.splits, C);
+  launch_reduce<1>(mode, grid, x, dy, save_mean, (double2*)ws, g);
+  TT_LAUNCH_CHECK();
+  BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws};
+  hipStream_t st = tt::stream();
+  if (mode == 0) bn_bwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 1) bn_bwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+  if (mode == 2) bn_bwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
+  TT_REQUIRE_INIT();
+  if (check_shape("tt_channel_sum_f32", N, K, HW)) return -1;
+  TT_REQUIRE(t && out, "tt_channel_sum_f32: null tensor pointer");
+  Geometry g;
+  int mode;
+  plan(N, K, HW, &g, &mode);
+  void* ws;
+  if (tt::workspace(sizeof(double2) * (size_t)K * g.splits, &ws)) return -1;
+  launch_reduce<2>(mode, dim3(g.splits, K), t, t, nullptr, (double2*)ws, g);
+  TT_LAUNCH_CHECK();
+  channel_sum_finish<<<K, tt::kWave, 0, tt::stream()>>>((const double2*)ws, out, g.splits);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

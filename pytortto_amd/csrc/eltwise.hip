@@ -1,0 +1,69 @@
+// Elementwise glue kernels (ReLU, residual add, gradient accumulation, fill): HBM-bound,
+// float4 grid-stride loops with a scalar tail.
+#include "tt_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill };
+
+template <int OP>
+__device__ __forceinline__ float apply1(float a, float b, float alpha) {
+  if (OP == kRelu) return fmaxf(a, 0.f);
+  if (OP == kReluBwd) return b > 0.f ? a : 0.f;  // a = dy, b = y
+  if (OP == kAdd) return a + b;
+  if (OP == kAxpy) return fmaf(alpha, a, b);      // a = v, b = acc
+  return alpha;                                    // kFill
+}
+
+template <int OP>
+__global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a, const float* __restrict__ b,
+                                                    float* __restrict__ out, float alpha, size_t n) {
+  constexpr bool kUseA = OP != kFill;
+  constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy;
+  const size_t n4 = n >> 2;
+  const size_t stride = (size_t)gridDim.x * kThreads;
+  for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
+    float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va, o;
+    if (kUseA) va = reinterpret_cast<const float4*>(a)[i];
+    if (kUseB) vb = reinterpret_cast<const float4*>(b)[i];
+    o.x = apply1<OP>(va.x, vb.x, alpha);
+    o.y = apply1<OP>(va.y, vb.y, alpha);
+    o.z = apply1<OP>(va.z, vb.z, alpha);
+    o.w = apply1<OP>(va.w, vb.w, alpha);
+    reinterpret_cast<float4*>(out)[i] = o;
+  }
+  // tail (n % 4 elements)
+  const size_t t = (n4 << 2) + (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (t < n) out[t] = apply1<OP>(kUseA ? a[t] : 0.f, kUseB ? b[t] : 0.f, alpha);
+}
+
+template <int OP>
+int run(const char* fn, const float* a, const float* b, float* out, float alpha, size_t n) {
+  TT_REQUIRE_INIT();
+  if (n == 0) return 0;
+  TT_REQUIRE(out != nullptr, "%s: null output pointer", fn);
+  size_t blocks = ((n >> 2) + kThreads - 1) / kThreads;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  eltwise<OP><<<(unsigned)blocks, kThreads, 0, tt::stream()>>>(a, b, out, alpha, n);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tt_relu_fwd_f32(const float* x, float* y, size_t n) { return run<kRelu>("tt_relu_fwd_f32", x, nullptr, y, 0.f, n); }
+int tt_relu_bwd_f32(const float* dy, const float* y, float* dx, size_t n) {
+  return run<kReluBwd>("tt_relu_bwd_f32", dy, y, dx, 0.f, n);
+}
+int tt_add_f32(const float* a, const float* b, float* out, size_t n) { return run<kAdd>("tt_add_f32", a, b, out, 0.f, n); }
+int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n) {
+  return run<kAxpy>("tt_axpy_f32", v, acc, acc, alpha, n);
+}
+int tt_fill_f32(float* dst, float value, size_t n) { return run<kFill>("tt_fill_f32", nullptr, nullptr, dst, value, n); }
+
+}  // extern "C"

@@ -1,0 +1,56 @@
+// Internal declarations shared by the translation units of libtortto_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/tortto_hip.h"
+
+namespace tt {
+
+// Records a message for tt_last_error() and returns a non-zero status.
+int fail(int code, const char* fmt, ...);
+int fail_hip(hipError_t e, const char* what, const char* file, int line);
+
+// The one stream every kernel of the library is enqueued on.
+hipStream_t stream();
+bool initialised();
+
+// Grow-only scratch memory owned by the library (split-K partial sums, repacked weights,
+// per-channel partial moments).  The pointer stays valid until the next call that asks for
+// more; work on the stream is ordered, so consecutive launches may reuse it.
+int workspace(size_t bytes, void** out);
+
+constexpr int kWave = 64;
+
+inline bool fits_i32(long long elems) { return elems >= 0 && elems < 2147483647LL; }
+
+// Unsigned division by a run-time constant without a divide instruction:
+// q = (umulhi(n, mul) + n) >> shift, valid for n < 2^31.
+struct FastDiv {
+  uint32_t mul;
+  uint32_t shift;
+  uint32_t d;
+};
+FastDiv make_fastdiv(uint32_t d);
+
+__device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv& f) {
+  return (uint32_t)(((uint64_t)__umulhi(n, f.mul) + n) >> f.shift);
+}
+
+}  // namespace tt
+
+#define TT_HIP(expr)                                                      \
+  do {                                                                    \
+    hipError_t _e = (expr);                                               \
+    if (_e != hipSuccess) return tt::fail_hip(_e, #expr, __FILE__, __LINE__); \
+  } while (0)
+
+#define TT_REQUIRE(cond, ...)                     \
+  do {                                            \
+    if (!(cond)) return tt::fail(-1, __VA_ARGS__); \
+  } while (0)
+
+#define TT_REQUIRE_INIT() TT_REQUIRE(tt::initialised(), "tt_init() has not been called")
+
+#define TT_LAUNCH_CHECK() TT_HIP(hipGetLastError())

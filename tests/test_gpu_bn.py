@@ -1,0 +1,151 @@
+"""GPU parity: BatchNorm2d training forward/backward through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+# outputs and running statistics: rtol 1e-5 (plus an absolute floor for values that cancel to ~0:
+# two correct float32 evaluations of (x-mean)/sd*gamma+beta differ by ~1 ulp of the larger term)
+RTOL = 1e-5
+
+
+def _close(got, ref, rtol=RTOL, atol_scale=2e-6, name=''):
+    ref = np.asarray(ref)
+    scale = float(np.abs(ref).max()) or 1.0
+    np.testing.assert_allclose(got, ref, rtol=rtol, atol=atol_scale * scale, err_msg=name)
+
+
+def _inputs(shape, seed=0):
+    np.random.seed(seed)
+    c = shape[1]
+    x = (2 + 3 * np.random.randn(*shape)).astype(np.float32)
+    gamma, beta = oracle.bn_affine_c4(c)
+    dy = np.random.randn(*shape).astype(np.float32)
+    return x, gamma, beta, dy
+
+
+SHAPES = [
+    (4, 3, 5, 5),        # flat scalar kernel, tiny
+    (2, 8, 1, 3),
+    (16, 5, 4, 4),       # flat float4 kernel
+    (8, 64, 14, 14),     # flat float4 (HW/4 = 49)
+    (8, 32, 7, 7),       # flat scalar, HW = 49
+    (6, 16, 16, 16),     # plane kernel, HW/4 = 64
+    (5, 7, 24, 20),      # plane kernel, ragged plane count per block
+    (64, 64, 28, 28),    # plane kernel with several splits per channel
+    (128, 4, 32, 32),    # few channels: maximum number of splits
+]
+
+
+@pytest.mark.parametrize('shape', SHAPES)
+def test_bn_train_fwd_bwd_matches_oracle(shape):
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    x, gamma, beta, dy = _inputs(shape)
+    c = shape[1]
+    rm0 = np.zeros(c, np.float32)
+    rv0 = np.ones(c, np.float32)
+    y_ref, saved, rm_ref, rv_ref = oracle.batch_norm_forward(x, gamma, beta, rm0, rv0, True, 0.1, 1e-5)
+    dx_ref, dg_ref, db_ref = oracle.batch_norm_backward(dy, x, gamma, saved)
+
+    xd, gd, bd, dyd = hiparray(x), hiparray(gamma), hiparray(beta), hiparray(dy)
+    y, mean, var_eps, sd, rm, rv = ops.bn_fwd_train(xd, gd, bd, hiparray(rm0), hiparray(rv0), 0.1, 1e-5)
+    dx, dg, db = ops.bn_bwd(xd, dyd, gd, mean, var_eps, sd)
+
+    _close(y.get(), y_ref, name='y')
+    _close(mean.get(), saved['mean'].ravel(), name='mean')
+    _close(var_eps.get(), saved['var'].ravel(), name='var+eps')
+    _close(sd.get(), saved['sd'].ravel(), name='sd')
+    _close(rm.get(), rm_ref, name='running_mean')
+    _close(rv.get(), rv_ref, name='running_var')
+    # gradients: long float32 reductions with cancellation on the CPU side -> compare against
+    # float64 truth as well and require the GPU to be at least as close as the oracle
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    y64, saved64, _, _ = oracle.batch_norm_forward(x64, gamma.astype(np.float64), beta.astype(np.float64),
+                                                   None, None, True, 0.1, 1e-5)
+    dx64, dg64, db64 = oracle.batch_norm_backward(dy64, x64, gamma.astype(np.float64), saved64)
+    for got, ref32, ref64, name in ((dx.get(), dx_ref, dx64, 'dx'), (dg.get(), dg_ref, dg64, 'dgamma'),
+                                    (db.get(), db_ref, db64, 'dbeta')):
+        scale = float(np.abs(ref64).max()) or 1.0
+        err_gpu = float(np.abs(got - ref64).max()) / scale
+        err_cpu = float(np.abs(ref32 - ref64).max()) / scale
+        assert err_gpu <= max(2 * err_cpu, 2e-6), (name, err_gpu, err_cpu)
+        _close(got, ref32, rtol=1e-4, atol_scale=1e-5, name=name)
+
+
+def test_bn_without_affine_and_without_running_stats():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    x, _, _, dy = _inputs((6, 16, 16, 16), seed=3)
+    y_ref, saved, rm_ref, rv_ref = oracle.batch_norm_forward(x, None, None, None, None, True, 0.1, 1e-5)
+    dx_ref, _, _ = oracle.batch_norm_backward(dy, x, None, saved, need=(True, False, False))
+    xd = hiparray(x)
+    y, mean, var_eps, sd, rm, rv = ops.bn_fwd_train(xd, None, None, None, None, 0.1, 1e-5)
+    assert rm is None and rv is None
+    dx, dg, db = ops.bn_bwd(xd, hiparray(dy), None, mean, var_eps, sd, need=(True, False, False))
+    assert dg is None and db is None
+    _close(y.get(), y_ref)
+    _close(dx.get(), dx_ref, rtol=1e-4, atol_scale=1e-5)
+
+
+def test_bn_running_stats_recurrence_three_steps():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    c = 16
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    rmd, rvd = hiparray(rm), hiparray(rv)
+    for step in range(3):
+        x, gamma, beta, _ = _inputs((6, c, 16, 16), seed=10 + step)
+        _, _, rm, rv = oracle.batch_norm_forward(x, gamma, beta, rm, rv, True, 0.3, 1e-5)
+        _, _, _, _, rmd, rvd = ops.bn_fwd_train(hiparray(x), hiparray(gamma), hiparray(beta), rmd, rvd, 0.3, 1e-5)
+    _close(rmd.get(), rm)
+    _close(rvd.get(), rv)
+
+
+def test_bn_eval_mode_matches_oracle():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    x, gamma, beta, dy = _inputs((6, 16, 16, 16), seed=5)
+    rm = np.linspace(1, 3, 16).astype(np.float32)
+    rv = np.linspace(4, 12, 16).astype(np.float32)
+    y_ref, saved, _, _ = oracle.batch_norm_forward(x, gamma, beta, rm, rv, False, 0.1, 1e-5)
+    dx_ref, dg_ref, db_ref = oracle.batch_norm_backward(dy, x, gamma, saved)
+    xd, gd = hiparray(x), hiparray(gamma)
+    y, mean, var_eps, sd = ops.bn_fwd_eval(xd, gd, hiparray(beta), hiparray(rm), hiparray(rv), 1e-5)
+    dx, dg, db = ops.bn_bwd(xd, hiparray(dy), gd, mean, var_eps, sd)
+    _close(y.get(), y_ref)
+    _close(dx.get(), dx_ref, rtol=1e-4, atol_scale=1e-5)
+    _close(dg.get(), dg_ref, rtol=1e-4, atol_scale=1e-5)
+    _close(db.get(), db_ref, rtol=1e-4, atol_scale=1e-5)
+
+
+def test_bn_large_mean_small_sigma_is_stable():
+    """|mean| >> sigma: a raw E[x^2]-E[x]^2 in float32 would lose every digit of the variance."""
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    np.random.seed(7)
+    x = (1000 + 0.5 * np.random.randn(8, 16, 16, 16)).astype(np.float32)
+    var64 = x.astype(np.float64).var((0, 2, 3))
+    _, mean, var_eps, _, _, _ = ops.bn_fwd_train(hiparray(x), None, None, None, None, 0.1, 0.0)
+    np.testing.assert_allclose(var_eps.get(), var64, rtol=1e-4)
+    np.testing.assert_allclose(mean.get(), x.astype(np.float64).mean((0, 2, 3)), rtol=1e-6)
+
+
+def test_bn_single_value_per_channel_is_an_error():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    with pytest.raises(RuntimeError, match='Expected more than 1 value per channel'):
+        ops.bn_fwd_train(hiparray(np.zeros((1, 3, 1, 1), np.float32)), None, None, None, None, 0.1, 1e-5)
+
+
+def test_channel_sum_matches_numpy():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    np.random.seed(2)
+    for shape in [(4, 6, 5, 5), (32, 32, 32, 32), (3, 5, 8, 4)]:
+        t = np.random.randn(*shape).astype(np.float32)
+        ref = t.astype(np.float64).sum((0, 2, 3))
+        got = ops.channel_sum(hiparray(t)).get()
+        np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(ref).max())
