@@ -1,0 +1,459 @@
+// Implicit-GEMM convolution on fp32 MFMA for gfx950: Conv2d forward, and the gather-form input
+// gradient that also serves as ConvTranspose2d forward.  NCHW float32, no im2col buffer in HBM.
+//
+// Per group the kernel computes   D[i, m] = sum_k  Wp[i, k] * G[k, m]   (+ bias[i])
+//   forward: i = output channel, m = (n, p, q) output pixel, k = (c, r, s),
+//            G[k, m] = x[n, c, p*sh + r*dh - ph, q*sw + s*dw - pw]  (0 outside the image)
+//   dgrad  : dx pixels are split into sh*sw stride-parity classes; inside a class every pixel
+//            has the same set of valid taps, so a class is again a dense GEMM with
+//            i = input channel, m = (n, h', w') with h = h'*sh + class_h, k = (ko, tr, ts),
+//            G[k, m] = dy[n, ko, ih_base(h') - tr*eh, iw_base(w') - ts*ew]
+//            (no zero-insertion, no wasted MACs at stride > 1; classes without a tap get bias/0).
+// Both are the same kernel: a pixel decomposes as (n, u, v), a reduction index k looks up
+// {element offset, row step, column step} in a small table read with scalar loads.
+//
+// Tiling: 256 threads = 4 waves; block tile BM x BN with BK = 16; each wave owns MT x NT
+// v_mfma_f32_32x32x2_f32 accumulators (rows = i from the weights, columns = pixels, so a
+// lane's 32 consecutive pixels store as 128 contiguous bytes of NCHW output).  Weights are
+// repacked once per call into k-quad-major float4 tiles [k/4][i][k%4]; the gathered operand is
+// written to LDS in the same layout, so every MFMA operand fetch is one ds_read_b128 that
+// yields four k-steps.  Global loads for chunk c+1 are issued before the MFMAs of chunk c
+// (register prefetch) and land in the other LDS buffer: one barrier per chunk.
+#include "tt_common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kBKQ = 4;          // k-quads per chunk (BK = 16)
+constexpr int kInvalid = -(1 << 20);
+
+// One entry per reduction index k (padded with never-valid entries to a whole chunk).
+struct KEntry {
+  int off;   // element offset added to the pixel's base offset
+  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit
+};
+
+typedef int intx2 __attribute__((ext_vector_type(2)));
+typedef const intx2 __attribute__((address_space(4))) * ConstKTab;   // constant address space: scalar (s_load) access
+
+struct Igemm {
+  const float* src;
+  const floatx4* wp;     // [G][KQ][Ipad] x 4 floats
+  const KEntry* ktab;    // [KQ*4]
+  const float* bias;     // [G*I] or null
+  float* out;
+  int I, Ipad, KQ, M;
+  tt::FastDiv divUV, divV;   // m -> (n, u, v)
+  int su, bh, sv, bw;        // ih0 = u*su + bh, iw0 = v*sv + bw
+  int Hlim, Wlim, srcRow;
+  int srcStrideN, srcStrideG;
+  int outStrideN, outStrideG, outStrideI, outRow;
+  int ou, ouh, ov, ovw;      // output row = u*ou + ouh, column = v*ov + ovw
+  int tilesI;                // row tiles per group
+  int tiles;                 // tilesI * pixel tiles
+};
+
+// ---- preparation kernels (tiny) --------------------------------------------------------------
+
+// Forward: Wp[g][kq][i][j] = w[g*I + i][4*kq + j]  (w rows are Kred = Cg*R*S long, 0 beyond).
+__global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp, int I, int Ipad, int Kred, int KQ) {
+  const int g = blockIdx.z, kq = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= Ipad) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (i < I) {
+    const float* row = w + ((size_t)g * I + i) * Kred;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (4 * kq + j < Kred) v[j] = row[4 * kq + j];
+  }
+  wp[((size_t)g * KQ + kq) * Ipad + i] = floatx4{v[0], v[1], v[2], v[3]};
+}
+
+// Input gradient, one stride-parity class: k = (ko*nTr + tr)*nTs + ts,
+// Wp[g][kq][c][j] = w[g*Kg + ko][c][r0 + tr*rstep][s0 + ts*sstep].
+struct PackDgrad {
+  int Kg, Cg, R, S, Ipad, Kred, KQ;
+  int nTr, nTs, r0, rstep, s0, sstep;
+};
+__global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ wp, PackDgrad a) {
+  const int g = blockIdx.z, kq = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.Ipad) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < a.Cg) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * kq + j;
+      if (k < a.Kred) {
+        const int ts = k % a.nTs, t = k / a.nTs;
+        const int tr = t % a.nTr, ko = t / a.nTr;
+        v[j] = w[((((size_t)g * a.Kg + ko) * a.Cg + c) * a.R + a.r0 + tr * a.rstep) * a.S + a.s0 + ts * a.sstep];
+      }
+    }
+  }
+  wp[((size_t)g * a.KQ + kq) * a.Ipad + c] = floatx4{v[0], v[1], v[2], v[3]};
+}
+
+// k -> {offset, steps}.  k = (a*TB + b)*TC + c:  off = a*sa + b*sb + c*sc, steps (b*stepH, c*stepW).
+struct KTabArgs {
+  int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
+};
+__global__ void build_ktab(KEntry* __restrict__ tab, KTabArgs a) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k >= a.Kpad) return;
+  KEntry e;
+  if (k < a.Kred) {
+    const int c = k % a.TC, t = k / a.TC;
+    const int b = t % a.TB, aa = t / a.TB;
+    e.off = aa * a.sa + b * a.sb + c * a.sc;
+    e.dhw = ((b * a.stepH) & 0xffff) | ((c * a.stepW) << 16);
+  } else {
+    e.off = 0;
+    e.dhw = (-16384) & 0xffff;   // row far above the image: never valid
+  }
+  tab[k] = e;
+}
+
+// ---- the GEMM kernel -----------------------------------------------------------------------------
+
+// Blocks are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles, row
+// tiles fastest, so blocks that share a pixel tile (same gathered operand) share an L2.
+__device__ __forceinline__ int xcd_remap(int b, int nb) {
+  const int q = nb >> 3, rem = nb & 7;
+  const int xcd = b & 7, idx = b >> 3;
+  return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
+}
+
+template <int WM, int WN, int MT, int NT>
+__global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
+  static_assert(WM * WN == 4, "four waves per block");
+  constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
+  constexpr int A_ITEMS = kBKQ * BM / kThreads, B_ITEMS = kBKQ * BN / kThreads;
+  static_assert(A_ITEMS >= 1 && B_ITEMS >= 1 && kThreads % BM == 0 && kThreads % BN == 0, "tile shape");
+  __shared__ floatx4 As[2][kBKQ][BM];
+  __shared__ floatx4 Bs[2][kBKQ][BN];
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int g = blockIdx.y;
+  const int tile = xcd_remap(blockIdx.x, p.tiles);
+  const int i0 = (tile % p.tilesI) * BM;
+  const int m0 = (tile / p.tilesI) * BN;
+
+  // gathered operand: this thread always loads the same pixel, for B_ITEMS k-quads per chunk
+  const int pix = tid % BN;
+  const int bq0 = __builtin_amdgcn_readfirstlane(tid / BN);   // first k-quad (wave-uniform)
+  int ih0 = kInvalid, iw0 = 0, base = 0;
+  {
+    const int m = m0 + pix;
+    if (m < p.M) {
+      const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
+      const uint32_t rem = (uint32_t)m - n * p.divUV.d;
+      const uint32_t u = tt::fd_div(rem, p.divV);
+      const uint32_t v = rem - u * p.divV.d;
+      ih0 = (int)u * p.su + p.bh;
+      iw0 = (int)v * p.sv + p.bw;
+      base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
+    }
+  }
+  const ConstKTab ktab = (ConstKTab)(uintptr_t)p.ktab;
+  const floatx4* __restrict__ wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
+  const int arow = tid % BM, aq0 = tid / BM;
+
+  floatx4 areg[A_ITEMS];
+  floatx4 breg[B_ITEMS];
+  bool bok[B_ITEMS][4];   // applied when the values are written to LDS, after the MFMAs
+
+  auto load_global = [&](int chunk) {
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) {
+      const int kq = chunk * kBKQ + aq0 + it * (kThreads / BM);
+      areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
+    }
+#pragma unroll
+    for (int it = 0; it < B_ITEMS; ++it) {
+      const int kq = chunk * kBKQ + bq0 + it * (kThreads / BN);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const intx2 e = ktab[kq * 4 + j];   // {off, dhw} of KEntry
+        const int ih = ih0 + (int)(short)(e.y & 0xffff);
+        const int iw = iw0 + (e.y >> 16);
+        const bool ok = (unsigned)ih < (unsigned)p.Hlim && (unsigned)iw < (unsigned)p.Wlim;
+        const uint32_t off = ok ? (uint32_t)(base + e.x) : 0u;
+        breg[it][j] = p.src[off];
+        bok[it][j] = ok;
+      }
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) As[buf][aq0 + it * (kThreads / BM)][arow] = areg[it];
+#pragma unroll
+    for (int it = 0; it < B_ITEMS; ++it)
+    {
+      floatx4 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
+      Bs[buf][bq0 + it * (kThreads / BN)][pix] = v;
+    }
+  };
+
+  floatx16 acc[MT][NT];
+#pragma unroll
+  for (int a = 0; a < MT; ++a)
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  const int chunks = p.KQ / kBKQ;
+  if (chunks > 0) {
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+  }
+  for (int c = 0; c < chunks; ++c) {
+    const int cur = c & 1;
+    // the last iteration re-fetches its own chunk (cache hit) into the idle buffer: keeping the
+    // loop body free of conditions lets the prefetch registers stay registers
+    load_global(min(c + 1, chunks - 1));
+    __builtin_amdgcn_sched_barrier(0);   // keep the prefetch ahead of the MFMAs it overlaps with
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      // lanes 0-31 take quad 2*kk, lanes 32-63 quad 2*kk+1: MFMA step j contracts k = 4*quad + j
+      floatx4 a[MT], b[NT];
+#pragma unroll
+      for (int x = 0; x < MT; ++x) a[x] = As[cur][kk * 2 + h][(wm * MT + x) * 32 + l32];
+#pragma unroll
+      for (int x = 0; x < NT; ++x) b[x] = Bs[cur][kk * 2 + h][(wn * NT + x) * 32 + l32];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int x = 0; x < MT; ++x)
+#pragma unroll
+          for (int y = 0; y < NT; ++y) {
+            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x][j], b[y][j], acc[x][y], 0, 0, 0);
+          }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*h + r%4, column l32
+  uint32_t obase[NT];
+  bool mok[NT];
+#pragma unroll
+  for (int y = 0; y < NT; ++y) {
+    const int m = m0 + (wn * NT + y) * 32 + l32;
+    mok[y] = m < p.M;
+    const uint32_t mm = mok[y] ? (uint32_t)m : 0u;
+    const uint32_t n = tt::fd_div(mm, p.divUV);
+    const uint32_t rem = mm - n * p.divUV.d;
+    const uint32_t u = tt::fd_div(rem, p.divV);
+    const uint32_t v = rem - u * p.divV.d;
+    obase[y] = (uint32_t)((int)n * p.outStrideN + g * p.outStrideG + ((int)u * p.ou + p.ouh) * p.outRow +
+                          (int)v * p.ov + p.ovw);
+  }
+#pragma unroll
+  for (int x = 0; x < MT; ++x) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (i < p.I) {
+        const float bz = p.bias ? p.bias[g * p.I + i] : 0.f;
+        const uint32_t ioff = (uint32_t)(i * p.outStrideI);
+#pragma unroll
+        for (int y = 0; y < NT; ++y)
+          if (mok[y]) p.out[obase[y] + ioff] = acc[x][y][r] + bz;
+      }
+    }
+  }
+}
+
+// ---- host side -------------------------------------------------------------------------------------
+
+int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+int gcd(int a, int b) { return b == 0 ? a : gcd(b, a % b); }
+
+struct TileChoice {
+  int bm, bn;
+};
+
+// 128x128 by default; 64 rows when a group has no more than 64 of them; 64x64 when the bigger
+// tiles would leave most of the 256 CUs idle.
+TileChoice choose_tile(int I, int M, int groups) {
+  TileChoice t;
+  if (I <= 64) {
+    t.bm = 64;
+    t.bn = 256;
+  } else {
+    t.bm = 128;
+    t.bn = 128;
+  }
+  const long long blocks = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn) * groups;
+  if (blocks < 256) {
+    t.bm = 64;
+    t.bn = 64;
+  }
+  return t;
+}
+
+int launch_igemm(Igemm& p, int groups, TileChoice t) {
+  p.tilesI = p.Ipad / t.bm;
+  p.tiles = p.tilesI * ceil_div(p.M, t.bn);
+  dim3 grid(p.tiles, groups);
+  hipStream_t st = tt::stream();
+  if (t.bm == 128 && t.bn == 128)
+    igemm_f32<2, 2, 2, 2><<<grid, kThreads, 0, st>>>(p);
+  else if (t.bm == 64 && t.bn == 256)
+    igemm_f32<1, 4, 2, 2><<<grid, kThreads, 0, st>>>(p);
+  else
+    igemm_f32<2, 2, 1, 1><<<grid, kThreads, 0, st>>>(p);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
+                 int dh, int dw, int groups, int P, int Q) {
+  TT_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0, "%s: sizes must be positive", fn);
+  TT_REQUIRE(sh > 0 && sw > 0 && dh > 0 && dw > 0 && ph >= 0 && pw >= 0, "%s: stride/dilation must be positive, padding non-negative", fn);
+  TT_REQUIRE(groups > 0 && C % groups == 0 && K % groups == 0, "%s: channels (%d, %d) not divisible by groups=%d", fn, C, K, groups);
+  TT_REQUIRE(P > 0 && Q > 0, "%s: empty output (%d x %d)", fn, P, Q);
+  TT_REQUIRE(groups <= 65535, "%s: more than 65535 groups are not supported", fn);
+  TT_REQUIRE((long long)H + 2 * ph + (long long)R * dh < 16384 && (long long)W + 2 * pw + (long long)S * dw < 16384 &&
+                 P < 16384 && Q < 16384,
+             "%s: spatial extents must stay below 16384", fn);
+  TT_REQUIRE(tt::fits_i32((long long)N * C * H * W) && tt::fits_i32((long long)N * K * P * Q) &&
+                 tt::fits_i32((long long)K * (C / groups) * R * S),
+             "%s: a tensor exceeds 2^31-1 elements", fn);
+  return 0;
+}
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+extern "C" {
+
+int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
+                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
+  const int P = (H + 2 * ph - dh * (R - 1) - 1) / sh + 1;
+  const int Q = (W + 2 * pw - dw * (S - 1) - 1) / sw + 1;
+  TT_REQUIRE(H + 2 * ph - dh * (R - 1) - 1 >= 0 && W + 2 * pw - dw * (S - 1) - 1 >= 0,
+             "tt_conv2d_fwd_f32: kernel (%d x %d, dilation %d x %d) larger than padded input (%d x %d)", R, S, dh, dw,
+             H + 2 * ph, W + 2 * pw);
+  if (check_common("tt_conv2d_fwd_f32", N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+  const int Cg = C / groups, Kg = K / groups;
+  const int Kred = Cg * R * S;
+  const int M = N * P * Q;
+  const TileChoice t = choose_tile(Kg, M, groups);
+  const int Ipad = ceil_div(Kg, t.bm) * t.bm;
+  const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
+
+  const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
+  const size_t tab_bytes = sizeof(KEntry) * (size_t)KQ * 4;
+  void* ws;
+  if (tt::workspace(wp_bytes + tab_bytes, &ws)) return -1;
+  floatx4* wp = (floatx4*)ws;
+  KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
+  hipStream_t st = tt::stream();
+  pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ);
+  TT_LAUNCH_CHECK();
+  KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
+  build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
+  TT_LAUNCH_CHECK();
+
+  Igemm p{};
+  p.src = x; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = y;
+  p.I = Kg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
+  p.divUV = tt::make_fastdiv((uint32_t)(P * Q));
+  p.divV = tt::make_fastdiv((uint32_t)Q);
+  p.su = sh; p.bh = -ph; p.sv = sw; p.bw = -pw;
+  p.Hlim = H; p.Wlim = W; p.srcRow = W;
+  p.srcStrideN = C * H * W; p.srcStrideG = Cg * H * W;
+  p.outStrideN = K * P * Q; p.outStrideG = Kg * P * Q; p.outStrideI = P * Q; p.outRow = Q;
+  p.ou = 1; p.ouh = 0; p.ov = 1; p.ovw = 0;
+  return launch_igemm(p, groups, t);
+}
+
+int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
+                        int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
+                        int Q) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
+  if (check_common("tt_conv2d_dgrad_f32", N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+  const int Cg = C / groups, Kg = K / groups;
+  const int gh = gcd(sh, dh), gw = gcd(sw, dw);
+  const int rstep = sh / gh, sstep = sw / gw;   // valid taps of a class: r0, r0+rstep, ...
+  const int eh = dh / gh, ew = dw / gw;          // dy row/column step per tap
+
+  // workspace: the largest class (all taps at stride 1) bounds every class
+  int max_taps_r = ceil_div(R, rstep), max_taps_s = ceil_div(S, sstep);
+  const int KQmax = ceil_div((long long)Kg * max_taps_r * max_taps_s, 4 * kBKQ) * kBKQ;
+  const int IpadMax = ceil_div(Cg, 128) * 128;
+  const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQmax * IpadMax, 256);
+  const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQmax * 4, 256);
+  const int classes = sh * sw;
+  TT_REQUIRE(classes <= 4096, "tt_conv2d_dgrad_f32: stride %d x %d not supported", sh, sw);
+  void* ws;
+  if (tt::workspace((wp_bytes + tab_bytes) * classes, &ws)) return -1;
+  hipStream_t st = tt::stream();
+
+  int slot = 0;
+  for (int ch = 0; ch < sh && ch < Hx; ++ch) {
+    // taps r with (ch + ph - r*dh) % sh == 0
+    int r0 = -1;
+    for (int r = 0; r < R && r < rstep; ++r)
+      if (((ch + ph - r * dh) % sh + sh) % sh == 0) { r0 = r; break; }
+    const int nTr = r0 < 0 ? 0 : ceil_div(R - r0, rstep);
+    const int U = ceil_div(Hx - ch, sh);
+    for (int cw = 0; cw < sw && cw < Wx; ++cw, ++slot) {
+      int s0 = -1;
+      for (int s = 0; s < S && s < sstep; ++s)
+        if (((cw + pw - s * dw) % sw + sw) % sw == 0) { s0 = s; break; }
+      const int nTs = s0 < 0 ? 0 : ceil_div(S - s0, sstep);
+      const int V = ceil_div(Wx - cw, sw);
+      const int Kred = Kg * nTr * nTs;
+      const int M = N * U * V;
+      const TileChoice t = choose_tile(Cg, M, groups);
+      const int Ipad = ceil_div(Cg, t.bm) * t.bm;
+      const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
+      floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
+      KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
+      Igemm p{};
+      if (KQ > 0) {
+        PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
+        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa);
+        TT_LAUNCH_CHECK();
+        KTabArgs ka{Kred, KQ * 4, nTr, nTs, P * Q, -eh * Q, -ew, -eh, -ew};
+        build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
+        TT_LAUNCH_CHECK();
+        // h = u*sh + ch reads dy row (h + ph - r0*dh)/sh = u + (ch + ph - r0*dh)/sh  (exact)
+        p.bh = (ch + ph - r0 * dh) / sh;   // numerator is a multiple of sh by choice of r0
+        p.bw = (cw + pw - s0 * dw) / sw;
+      }
+      p.src = dy; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.I = Cg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
+      p.divUV = tt::make_fastdiv((uint32_t)(U * V));
+      p.divV = tt::make_fastdiv((uint32_t)V);
+      p.su = 1; p.sv = 1;
+      p.Hlim = P; p.Wlim = Q; p.srcRow = Q;
+      p.srcStrideN = K * P * Q; p.srcStrideG = Kg * P * Q;
+      p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
+      p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
+      if (launch_igemm(p, groups, t)) return -1;
+    }
+  }
+  return 0;
+}
+
+}  // extern "C"

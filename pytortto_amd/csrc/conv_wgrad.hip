@@ -1,0 +1,273 @@
+// Weight gradient of Conv2d on fp32 MFMA for gfx950 (NCHW float32).
+//
+// Per group:  dw[i, j] = sum_m  dy[m, i] * x~[m, j],   i = output channel, j = (c, r, s),
+// m = (n, p, q) running over all N*P*Q output pixels (the reduction).  The output is small and
+// the reduction long (up to ~8e5), so the reduction is split over blockIdx.z into `splits`
+// contiguous ranges of 32-pixel chunks; each split writes an fp32 partial tile to the
+// workspace and a second kernel adds the partials in a fixed order in float64
+// (deterministic, and more accurate than one long fp32 accumulation).
+//
+// Both operands are contiguous along the reduction index in NCHW memory, so lanes run along
+// pixels for coalesced loads and the LDS tiles are [row][pixel] with a 4-float pad: an MFMA
+// operand fetch is one ds_read_b128 holding four reduction steps, conflict-free because
+// consecutive rows start 36 floats apart.  v_mfma_f32_32x32x2_f32 rows = output channels,
+// columns = (c,r,s), so 32 lanes store 128 contiguous bytes of dw.
+#include "tt_common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kBK = 32;        // pixels per chunk
+constexpr int kLd = kBK + 4;   // padded LDS row (floats)
+constexpr int kInvalid = -(1 << 20);
+
+struct Wgrad {
+  const float* x;
+  const float* dy;
+  float* out;            // dw (splits == 1) or workspace [splits][G][Kg][J]
+  int Kg, J, M;          // rows, columns (Cg*R*S), reduction length
+  int chunks, chunksPerSplit;
+  tt::FastDiv divPQ, divQ, divRS, divS;
+  int sh, sw, ph, pw, dh, dw;
+  int H, W, HW;
+  int xStrideN, xStrideG;     // C*H*W, Cg*H*W
+  int dyStrideN, dyStrideG;   // K*P*Q, Kg*P*Q
+  int PQ;
+  int tilesI;
+  size_t outStrideSplit;      // G*Kg*J
+};
+
+template <int WM, int WN, int MT, int NT>
+__global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
+  static_assert(WM * WN == 4, "four waves per block");
+  constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
+  constexpr int A_ROWS = BM / 8, B_ROWS = BN / 8;   // rows per thread (8 row groups of 32 lanes)
+  __shared__ __attribute__((aligned(16))) float As[BM][kLd];
+  __shared__ __attribute__((aligned(16))) float Bs[BN][kLd];
+  __shared__ int2 jtab[BN];   // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int g = blockIdx.y, split = blockIdx.z;
+  const int i0 = (blockIdx.x % p.tilesI) * BM;
+  const int j0 = (blockIdx.x / p.tilesI) * BN;
+
+  if (tid < BN) {
+    const int j = j0 + tid;
+    int2 e = make_int2(0, (-16384) & 0xffff);   // column beyond J: never valid
+    if (j < p.J) {
+      const uint32_t c = tt::fd_div((uint32_t)j, p.divRS);
+      const uint32_t rs = (uint32_t)j - c * p.divRS.d;
+      const uint32_t r = tt::fd_div(rs, p.divS);
+      const uint32_t s = rs - r * p.divS.d;
+      e.x = (int)c * p.HW + (int)r * p.dh * p.W + (int)s * p.dw;
+      e.y = (((int)r * p.dh) & 0xffff) | (((int)s * p.dw) << 16);
+    }
+    jtab[tid] = e;
+  }
+
+  const int px = tid & 31, rg = tid >> 5;   // this thread's pixel inside a chunk, and row group
+  const float* __restrict__ dyg = p.dy + (size_t)g * p.dyStrideG;
+  const float* __restrict__ xg = p.x + (size_t)g * p.xStrideG;
+
+  float areg[A_ROWS], breg[B_ROWS];
+  bool aok = false;
+  uint32_t bok = 0;   // bit t: breg[t] is inside the image (applied when written to LDS)
+  int2 jreg[B_ROWS];
+
+  const int c_begin = split * p.chunksPerSplit;
+  const int c_end = min(p.chunks, c_begin + p.chunksPerSplit);
+
+  auto load_global = [&](int chunk) {
+    const int m = chunk * kBK + px;
+    int ih0 = kInvalid, iw0 = 0, xbase = 0, dybase = 0;
+    const bool mok = m < p.M;
+    aok = mok;
+    bok = 0;
+    if (mok) {
+      const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
+      const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
+      const uint32_t pp = tt::fd_div(pq, p.divQ);
+      const uint32_t qq = pq - pp * p.divQ.d;
+      ih0 = (int)pp * p.sh - p.ph;
+      iw0 = (int)qq * p.sw - p.pw;
+      xbase = (int)n * p.xStrideN + ih0 * p.W + iw0;
+      dybase = (int)n * p.dyStrideN + (int)pq;
+    }
+#pragma unroll
+    for (int t = 0; t < A_ROWS; ++t) {
+      const int i = i0 + rg + 8 * t;
+      const bool ok = mok && i < p.Kg;
+      areg[t] = dyg[ok ? (uint32_t)(dybase + i * p.PQ) : 0u];
+    }
+#pragma unroll
+    for (int t = 0; t < B_ROWS; ++t) {
+      const int2 e = jreg[t];
+      const int ih = ih0 + (int)(short)(e.y & 0xffff);
+      const int iw = iw0 + (e.y >> 16);
+      const bool ok = (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+      breg[t] = xg[ok ? (uint32_t)(xbase + e.x) : 0u];
+      bok |= ok ? (1u << t) : 0u;
+    }
+  };
+  auto store_lds = [&]() {
+    // rows beyond Kg / columns beyond J may hold anything (never stored); pixels beyond M and
+    // taps outside the image must be exactly zero: AND with an all-ones / all-zeros word
+    const int amask = aok ? -1 : 0;
+#pragma unroll
+    for (int t = 0; t < A_ROWS; ++t) As[rg + 8 * t][px] = __int_as_float(__float_as_int(areg[t]) & amask);
+#pragma unroll
+    for (int t = 0; t < B_ROWS; ++t) {
+      const int bmask = ((int)(bok << (31 - t))) >> 31;
+      Bs[rg + 8 * t][px] = __int_as_float(__float_as_int(breg[t]) & bmask);
+    }
+  };
+
+  floatx16 acc[MT][NT];
+#pragma unroll
+  for (int a = 0; a < MT; ++a)
+#pragma unroll
+    for (int b = 0; b < NT; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  __syncthreads();   // jtab
+#pragma unroll
+  for (int t = 0; t < B_ROWS; ++t) jreg[t] = jtab[rg + 8 * t];
+
+  if (c_begin < c_end) load_global(c_begin);
+  for (int c = c_begin; c < c_end; ++c) {
+    store_lds();
+    __syncthreads();
+    load_global(min(c + 1, c_end - 1));   // in flight while the MFMAs below run (last: harmless re-fetch)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < kBK / 8; ++kk) {
+      floatx4 a[MT], b[NT];
+#pragma unroll
+      for (int xx = 0; xx < MT; ++xx)
+        a[xx] = *reinterpret_cast<const floatx4*>(&As[(wm * MT + xx) * 32 + l32][kk * 8 + 4 * h]);
+#pragma unroll
+      for (int yy = 0; yy < NT; ++yy)
+        b[yy] = *reinterpret_cast<const floatx4*>(&Bs[(wn * NT + yy) * 32 + l32][kk * 8 + 4 * h]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int xx = 0; xx < MT; ++xx)
+#pragma unroll
+          for (int yy = 0; yy < NT; ++yy) {
+            acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[xx][j], b[yy][j], acc[xx][yy], 0, 0, 0);
+          }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();   // every wave is done reading before the next chunk overwrites the tiles
+  }
+
+  float* __restrict__ out = p.out + (size_t)split * p.outStrideSplit + (size_t)g * p.Kg * p.J;
+#pragma unroll
+  for (int yy = 0; yy < NT; ++yy) {
+    const int j = j0 + (wn * NT + yy) * 32 + l32;
+    if (j >= p.J) continue;
+#pragma unroll
+    for (int xx = 0; xx < MT; ++xx)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = i0 + (wm * MT + xx) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (i < p.Kg) out[(size_t)i * p.J + j] = acc[xx][yy][r];
+      }
+  }
+}
+
+// dw[e] = sum over splits of partial[s][e], added in split order in float64.
+__global__ __launch_bounds__(kThreads) void wgrad_reduce(const float* __restrict__ partial, float* __restrict__ dw,
+                                                         size_t elems, int splits) {
+  const size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
+  if (e >= elems) return;
+  double s = 0.0;
+  for (int k = 0; k < splits; ++k) s += (double)partial[(size_t)k * elems + e];
+  dw[e] = (float)s;
+}
+
+int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+}  // namespace
+
+extern "C" {
+
+int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
+                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+  TT_REQUIRE_INIT();
+  const char* fn = "tt_conv2d_wgrad_f32";
+  TT_REQUIRE(x && dy && dw, "%s: null tensor pointer", fn);
+  TT_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0 && P > 0 && Q > 0, "%s: sizes must be positive", fn);
+  TT_REQUIRE(sh > 0 && sw > 0 && dh > 0 && dw_ > 0 && ph >= 0 && pw >= 0, "%s: stride/dilation must be positive, padding non-negative", fn);
+  TT_REQUIRE(groups > 0 && groups <= 65535 && C % groups == 0 && K % groups == 0, "%s: channels (%d, %d) not divisible by groups=%d", fn, C, K, groups);
+  TT_REQUIRE(H + 2 * ph + R * dh < 16384 && W + 2 * pw + S * dw_ < 16384, "%s: spatial extents must stay below 16384", fn);
+  TT_REQUIRE(tt::fits_i32((long long)N * C * H * W) && tt::fits_i32((long long)N * K * P * Q) &&
+                 tt::fits_i32((long long)K * (C / groups) * R * S),
+             "%s: a tensor exceeds 2^31-1 elements", fn);
+  const int Cg = C / groups, Kg = K / groups;
+  const int J = Cg * R * S;
+  const long long Mll = (long long)N * P * Q;
+  const int M = (int)Mll;
+
+  int bm = 128, bn = 128;
+  if (Kg <= 64) bm = 64;
+  if (J <= 64) bn = 64;
+  const int tilesI = ceil_div(Kg, bm), tilesJ = ceil_div(J, bn);
+  const long long tiles = (long long)tilesI * tilesJ * groups;
+  const int chunks = ceil_div(M, kBK);
+  // enough blocks for ~3 per CU, but at least 8 chunks (256 pixels) of work per split
+  int splits = (int)((768 + tiles - 1) / tiles);
+  if (splits > chunks / 8) splits = chunks / 8;
+  if (splits < 1) splits = 1;
+  if (splits > 4096) splits = 4096;
+  int cps = ceil_div(chunks, splits);
+  splits = ceil_div(chunks, cps);
+
+  const size_t elems = (size_t)groups * Kg * J;
+  float* target = dw;
+  if (splits > 1) {
+    void* ws;
+    if (tt::workspace(sizeof(float) * elems * splits, &ws)) return -1;
+    target = (float*)ws;
+  }
+  Wgrad p{};
+  p.x = x; p.dy = dy; p.out = target;
+  p.Kg = Kg; p.J = J; p.M = M;
+  p.chunks = chunks; p.chunksPerSplit = cps;
+  p.divPQ = tt::make_fastdiv((uint32_t)(P * Q));
+  p.divQ = tt::make_fastdiv((uint32_t)Q);
+  p.divRS = tt::make_fastdiv((uint32_t)(R * S));
+  p.divS = tt::make_fastdiv((uint32_t)S);
+  p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw; p.dh = dh; p.dw = dw_;
+  p.H = H; p.W = W; p.HW = H * W;
+  p.xStrideN = C * H * W; p.xStrideG = Cg * H * W;
+  p.dyStrideN = K * P * Q; p.dyStrideG = Kg * P * Q;
+  p.PQ = P * Q;
+  p.tilesI = tilesI;
+  p.outStrideSplit = elems;
+  dim3 grid(tilesI * tilesJ, groups, splits);
+  hipStream_t st = tt::stream();
+  if (bm == 128 && bn == 128)
+    wgrad_f32<2, 2, 2, 2><<<grid, kThreads, 0, st>>>(p);
+  else if (bm == 64 && bn == 128)
+    wgrad_f32<2, 2, 1, 2><<<grid, kThreads, 0, st>>>(p);
+  else if (bm == 128 && bn == 64)
+    wgrad_f32<2, 2, 2, 1><<<grid, kThreads, 0, st>>>(p);
+  else
+    wgrad_f32<2, 2, 1, 1><<<grid, kThreads, 0, st>>>(p);
+  TT_LAUNCH_CHECK();
+  if (splits > 1) {
+    wgrad_reduce<<<ceil_div((long long)elems, kThreads), kThreads, 0, st>>>(target, dw, elems, splits);
+    TT_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
+}  // extern "C"

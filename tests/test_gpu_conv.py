@@ -1,0 +1,129 @@
+"""GPU parity: Conv2d / ConvTranspose2d forward, dgrad, wgrad through the C ABI vs the CPU oracle.
+
+Tolerance (fp32): allclose(rtol=1e-4, atol=1e-5) against the oracle for forward/dgrad.  For
+weight/bias gradients -- reductions over N*P*Q terms -- two correct float32 evaluations differ
+on near-zero entries by more than an element-wise rtol allows (the reference's own notebook
+check used rtol=1e-3 for them), so those use atol scaled by the tensor's magnitude, and every
+tensor is additionally required to be as close to a float64 evaluation as the oracle itself.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from tests.cases import CONV_CASES, CONVT_CASES
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(name, got, ref32, ref64, reduction=False):
+    scale = float(np.abs(ref64).max()) or 1.0
+    err_gpu = float(np.abs(got - ref64).max()) / scale
+    err_cpu = float(np.abs(ref32 - ref64).max()) / scale
+    assert err_gpu <= max(3 * err_cpu, 5e-6), f'{name}: gpu err {err_gpu:.3g} vs oracle err {err_cpu:.3g}'
+    atol = 1e-5 * max(1.0, scale) if reduction else 1e-5
+    np.testing.assert_allclose(got, ref32, rtol=1e-4, atol=atol, err_msg=name)
+
+
+def _run_conv(case, seed=0, bias=True):
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((n, c, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((k, c // g, r, s)) / np.sqrt(c // g * r * s)).astype(np.float32)
+    b = rng.standard_normal(k).astype(np.float32) if bias else None
+    y32, xpad = oracle.convolution_forward(x, w, b, st, pd, dl, g)
+    gy = rng.standard_normal(y32.shape).astype(np.float32)
+    dx32, dw32, db32 = oracle.convolution_backward(gy, x, xpad, w, st, pd, dl, g)
+    x64, w64, gy64 = x.astype(np.float64), w.astype(np.float64), gy.astype(np.float64)
+    y64, xpad64 = oracle.convolution_forward(x64, w64, None if b is None else b.astype(np.float64), st, pd, dl, g)
+    dx64, dw64, db64 = oracle.convolution_backward(gy64, x64, xpad64, w64, st, pd, dl, g)
+
+    xd, wd, gyd = hiparray(x), hiparray(w), hiparray(gy)
+    bd = None if b is None else hiparray(b)
+    y = ops.conv2d_fwd(xd, wd, bd, st, pd, dl, g)
+    assert y.shape == y32.shape
+    dx = ops.conv2d_dgrad(gyd, wd, None, (h, w_), st, pd, dl, g)
+    dw = ops.conv2d_wgrad(xd, gyd, w.shape, st, pd, dl, g)
+    db = ops.channel_sum(gyd)
+    _check('y', y.get(), y32, y64)
+    _check('dx', dx.get(), dx32, dx64)
+    _check('dw', dw.get(), dw32, dw64, reduction=True)
+    _check('db', db.get(), db32, db64, reduction=True)
+
+
+@pytest.mark.parametrize('case', CONV_CASES)
+def test_conv_small_geometries(case):
+    _run_conv(case)
+
+
+# shapes that exercise every tile configuration, ragged tiles, split reductions and groups
+TILE_CASES = [
+    (32, 16, 32, 32, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # the CPU-runnable baseline config
+    (4, 64, 28, 28, 64, 1, 1, (1, 1), (0, 0), (1, 1), 1),       # 64-row tile x 256 pixels
+    (4, 64, 28, 28, 256, 1, 1, (1, 1), (0, 0), (1, 1), 1),      # 128x128 tiles
+    (3, 96, 15, 15, 200, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # ragged rows (200) and pixels (675)
+    (4, 128, 28, 28, 128, 3, 3, (2, 2), (1, 1), (1, 1), 1),     # stride 2: four parity classes in dgrad
+    (4, 256, 14, 14, 512, 1, 1, (2, 2), (0, 0), (1, 1), 1),     # strided 1x1 shortcut
+    (8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1),        # stem: C=3, Kred=147 (not a multiple of 4)
+    (2, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # small M, long reduction
+    (4, 64, 20, 20, 96, 3, 3, (1, 1), (2, 2), (2, 2), 4),       # groups + dilation
+    (128, 4, 64, 64, 16, 3, 2, (1, 3), (2, 3), (1, 2), 2),      # the reference notebook's configuration
+]
+
+
+@pytest.mark.parametrize('case', TILE_CASES)
+def test_conv_tile_configurations(case):
+    _run_conv(case, seed=1)
+
+
+def test_conv_without_bias():
+    _run_conv((2, 4, 8, 8, 6, 3, 3, (1, 1), (1, 1), (1, 1), 1), bias=False)
+
+
+CONVT_TILE_CASES = [
+    (16, 100, 1, 1, 512, 4, 4, (1, 1), (0, 0), (0, 0), (1, 1), 1),   # DCGAN layer 1 (reduced batch)
+    (8, 256, 8, 8, 128, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),    # DCGAN upsampling layer
+    (8, 64, 16, 16, 3, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),     # DCGAN last layer: 3 output channels
+]
+
+
+@pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES)
+def test_conv_transpose_forward_backward(case):
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    n, ci, h, w_, co, r, s, st, pd, op, dl, g = case
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((n, ci, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((ci, co // g, r, s)) / np.sqrt(ci // g * r * s)).astype(np.float32)
+    b = rng.standard_normal(co).astype(np.float32)
+    y32 = oracle.transposed_convolution_forward(x, w, b, st, pd, op, dl, g)
+    gy = rng.standard_normal(y32.shape).astype(np.float32)
+    dx32, dw32, db32 = oracle.transposed_convolution_backward(gy, x, w, st, pd, dl, g)
+    x64, w64, gy64 = x.astype(np.float64), w.astype(np.float64), gy.astype(np.float64)
+    y64 = oracle.transposed_convolution_forward(x64, w64, b.astype(np.float64), st, pd, op, dl, g)
+    dx64, dw64, db64 = oracle.transposed_convolution_backward(gy64, x64, w64, st, pd, dl, g)
+
+    xd, wd, gyd = hiparray(x), hiparray(w), hiparray(gy)
+    # forward = input gradient of the convolution whose weight is w: "K" = C_in, "C" = C_out
+    y = ops.conv2d_dgrad(xd, wd, hiparray(b), y32.shape[-2:], st, pd, dl, g)
+    assert y.shape == y32.shape
+    dx = ops.conv2d_fwd(gyd, wd, None, st, pd, dl, g)
+    assert dx.shape == x.shape
+    dw = ops.conv2d_wgrad(gyd, xd, w.shape, st, pd, dl, g)
+    db = ops.channel_sum(gyd)
+    _check('y', y.get(), y32, y64)
+    _check('dx', dx.get(), dx32, dx64)
+    _check('dw', dw.get(), dw32, dw64, reduction=True)
+    _check('db', db.get(), db32, db64, reduction=True)
+
+
+def test_conv_rejects_bad_arguments():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    x = hiparray(np.zeros((1, 4, 4, 4), np.float32))
+    w = hiparray(np.zeros((4, 4, 3, 3), np.float32))
+    with pytest.raises(RuntimeError):
+        ops.conv2d_fwd(x, w, None, (1, 1), (0, 0), (1, 1), 3)      # channels not divisible by groups
+    with pytest.raises(RuntimeError):
+        ops.conv2d_fwd(x, w, None, (1, 1), (0, 0), (2, 2), 1)      # dilated kernel larger than the input
