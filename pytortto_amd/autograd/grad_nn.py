@@ -1,0 +1,191 @@
+"""The hot-path autograd functions with the reference's names, arguments and error behaviour
+(``src/tortto/autograd/grad_nn.py``): ``Convolution`` (:684-734), ``TransposedConvolution``
+(:737-779), ``BatchNorm`` (:907-989) and ``Relu`` (:33-69).
+
+Where the reference evaluates NumPy/CuPy expressions, these call ``libtortto_hip.so`` through
+``pytortto_amd.ops``.  Only device tensors (``hiparray``) are computed here: host tensors stay
+with tortto's own NumPy path, and are refused rather than silently computed some other way.
+"""
+from math import prod
+
+import numpy as np
+
+from .. import ops
+from ..xparray import hiparray
+from .function import Function
+from .helper import build_links, inplace_precheck, inplace_update
+
+
+def _device_only(name, data):
+    if data.__class__ is not hiparray:
+        raise RuntimeError(f'{name}: pytortto_amd implements the device (HIP) path only and got a host '
+                           f'{data.__class__.__name__}; move the tensors with .cuda() first '
+                           f'(host tensors belong to tortto\'s NumPy path)')
+
+
+class Convolution(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, xt1, xt2 = inputs   # input, weight, bias
+        xd0, xd1 = xt0.data, xt1.data
+        xd2 = None if xt2 is None else xt2.data
+        stride, padding = params['stride'], params['padding']
+        dilation, groups = params['dilation'], params['groups']
+        if xd0.__class__ is not xd1.__class__:
+            raise RuntimeError(f'Input type ({xd0.__class__.__name__}) and weight type '
+                               f'({xd1.__class__.__name__}) should be the same')
+        if xd2 is not None and xd0.__class__ is not xd2.__class__:
+            raise RuntimeError(f'Input type ({xd0.__class__.__name__}) and bias type '
+                               f'({xd2.__class__.__name__}) should be the same')
+        if xd0.ndim != 4:
+            raise RuntimeError(f'Expected 3D (unbatched) or 4D (batched) input to conv2d, '
+                               f'but got input of size: {xd0.shape}')
+        if groups * xd1.shape[-3] != xd0.shape[-3]:
+            raise RuntimeError(f'Given groups={groups}, weight of size {xd1.shape}, '
+                               f'expected input{xd0.shape} to have {groups * xd1.shape[-3]} channels, '
+                               f'but got {xd0.shape[-3]} channels instead')
+        _device_only('Convolution', xd0)
+        yd0 = ops.conv2d_fwd(xd0, xd1, xd2, stride, padding, dilation, groups)
+        yt0 = build_links(yd0, grad_fn=ctx)
+        # the reference also keeps a zero-padded copy of the input for the weight gradient
+        # (grad_nn.py:714); the kernels address padding implicitly, so the input itself suffices
+        ctx.save_for_backward(xt0, xt1)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        xd0, xd1 = ctx.saved_tensors
+        stride, padding = ctx.params['stride'], ctx.params['padding']
+        dilation, groups = ctx.params['dilation'], ctx.params['groups']
+        grad0 = grad1 = grad2 = None
+        if ctx.needs_input_grad[2]:
+            grad2 = ops.channel_sum(gd0)
+        if ctx.needs_input_grad[1]:
+            grad1 = ops.conv2d_wgrad(xd0, gd0, xd1.shape, stride, padding, dilation, groups)
+        if ctx.needs_input_grad[0]:
+            grad0 = ops.conv2d_dgrad(gd0, xd1, None, xd0.shape[-2:], stride, padding, dilation, groups)
+        return grad0, grad1, grad2
+
+
+class TransposedConvolution(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, xt1, xt2 = inputs   # input, weight [C_in, C_out/groups, R, S], bias
+        xd0, xd1 = xt0.data, xt1.data
+        stride, padding = params['stride'], params['padding']
+        dilation, groups = params['dilation'], params['groups']
+        output_padding = params['output_padding']
+        if xd0.ndim != 4:
+            raise RuntimeError(f'Expected 3D (unbatched) or 4D (batched) input to conv_transpose2d, '
+                               f'but got input of size: {xd0.shape}')
+        if xd1.shape[-4] != xd0.shape[-3]:
+            raise RuntimeError(f'Given transposed=1, weight of size {xd1.shape}, '
+                               f'expected input {xd0.shape} to have {xd1.shape[-4]} channels, '
+                               f'but got {xd0.shape[-3]} channels instead')
+        _device_only('TransposedConvolution', xd0)
+        _device_only('TransposedConvolution', xd1)
+        oph = output_padding[0]
+        opw = oph if len(output_padding) == 1 else output_padding[1]
+        r, s = xd1.shape[-2:]
+        hy = (xd0.shape[-2] - 1) * stride[0] - 2 * padding[0] + dilation[0] * (r - 1) + oph + 1
+        wy = (xd0.shape[-1] - 1) * stride[1] - 2 * padding[1] + dilation[1] * (s - 1) + opw + 1
+        # the forward pass is the input gradient of the convolution that has this weight
+        yd0 = ops.conv2d_dgrad(xd0, xd1, None if xt2 is None else xt2.data, (hy, wy),
+                               stride, padding, dilation, groups)
+        yt0 = build_links(yd0, grad_fn=ctx)
+        ctx.save_for_backward(xt0, xt1)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        xd0, xd1 = ctx.saved_tensors
+        stride, padding = ctx.params['stride'], ctx.params['padding']
+        dilation, groups = ctx.params['dilation'], ctx.params['groups']
+        grad0 = grad1 = grad2 = None
+        if ctx.needs_input_grad[2]:
+            grad2 = ops.channel_sum(gd0)
+        if ctx.needs_input_grad[1]:
+            grad1 = ops.conv2d_wgrad(gd0, xd0, xd1.shape, stride, padding, dilation, groups)
+        if ctx.needs_input_grad[0]:
+            # Always the padded convolution.  The reference drops the padding here when the
+            # weight needs no gradient (grad_nn.py:778), which is wrong for padding != 0.
+            grad0 = ops.conv2d_fwd(gd0, xd1, None, stride, padding, dilation, groups)
+        return grad0, grad1, grad2
+
+
+def _verify_batch_size(size):
+    """grad_nn.py:899-904"""
+    if prod((size[0],) + tuple(size[2:])) == 1:
+        raise ValueError(f'Expected more than 1 value per channel when training, got input size {size}')
+
+
+class BatchNorm(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, xt1, xt2 = inputs   # input, weight, bias
+        xd0 = xt0.data
+        running_mean, running_var = params['running_mean'], params['running_var']
+        training, momentum, eps = params['training'], params['momentum'], params['eps']
+        _device_only('BatchNorm', xd0)
+        gamma = None if xt1 is None else xt1.data
+        beta = None if xt2 is None else xt2.data
+        have_running = running_mean is not None and running_var is not None
+        cshape = (xd0.shape[1],) + (1,) * (xd0.ndim - 2)
+        if training:
+            _verify_batch_size(xd0.shape)
+            yd0, mean, var_eps, sd, new_rm, new_rv = ops.bn_fwd_train(
+                xd0, gamma, beta, running_mean.data if have_running else None,
+                running_var.data if have_running else None, momentum, eps)
+            if have_running:            # the buffers are re-bound to new arrays (grad_nn.py:929-930)
+                running_mean.data = new_rm
+                running_var.data = new_rv
+        elif have_running:
+            yd0, mean, var_eps, sd = ops.bn_fwd_eval(xd0, gamma, beta, running_mean.data, running_var.data, eps)
+        else:
+            yd0, mean, var_eps, sd, _, _ = ops.bn_fwd_train(xd0, gamma, beta, None, None, 0.0, eps)
+        yt0 = build_links(yd0, grad_fn=ctx)
+        ctx.save_for_backward(xt0, xt1)
+        ctx.params = {'axis': (0,) + tuple(range(2, xd0.ndim)), 'shape': (xd0.shape[0],) + xd0.shape[2:],
+                      'mean': mean.reshape(cshape), 'var': var_eps.reshape(cshape), 'sd': sd.reshape(cshape)}
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        xd0, xd1 = ctx.saved_tensors
+        p = ctx.params
+        grad0, grad1, grad2 = ops.bn_bwd(xd0, gd0, xd1, p['mean'], p['var'], p['sd'], need=ctx.needs_input_grad)
+        return grad0, grad1, grad2
+
+
+class Relu(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, = inputs
+        xd0 = xt0.data
+        inplace = params['inplace']
+        if xd0.__class__ is hiparray:
+            if inplace:
+                inplace_precheck(xt0)
+                ops.relu_fwd(xd0, out=xd0)
+                yt0 = inplace_update(xt0, ctx)
+            else:
+                yt0 = build_links(ops.relu_fwd(xd0), grad_fn=ctx)
+        elif inplace:
+            inplace_precheck(xt0)
+            np.maximum(xd0, 0, out=xd0)
+            yt0 = inplace_update(xt0, ctx)
+        else:
+            yt0 = build_links(np.maximum(xd0, 0), grad_fn=ctx)
+        ctx.save_for_backward(yt0)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        yd0, = ctx.saved_tensors
+        if yd0.__class__ is hiparray:
+            return ops.relu_bwd(gd0, yd0)
+        return gd0 * (yd0 > 0)

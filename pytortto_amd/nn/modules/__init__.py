@@ -1,0 +1,7 @@
+from .module import Module
+from .conv import Conv2d, ConvTranspose2d
+from .batchnorm import BatchNorm1d, BatchNorm2d, BatchNorm3d
+from .container import Sequential
+from .activation import ReLU
+
+__all__ = ['Module', 'Conv2d', 'ConvTranspose2d', 'BatchNorm1d', 'BatchNorm2d', 'BatchNorm3d', 'Sequential', 'ReLU']

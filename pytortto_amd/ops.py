@@ -131,9 +131,9 @@ def bn_bwd(x, dy, gamma, mean, var_eps, sd, need=(True, True, True)):
 
 # ---- elementwise glue ----------------------------------------------------------------------------
 
-def relu_fwd(x):
+def relu_fwd(x, out=None):
     _f32(x)
-    y = hiparray.empty(x.shape)
+    y = hiparray.empty(x.shape) if out is None else out
     _hip.call('tt_relu_fwd_f32', x.ptr, y.ptr, x.size)
     return y
 

@@ -1,0 +1,161 @@
+"""GPU parity at the module level: nn.Conv2d / nn.ConvTranspose2d / nn.BatchNorm2d with
+``.cuda()`` semantics and autograd, against the CPU oracle on identical seeded inputs."""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, ref, rtol=1e-4, atol=1e-5, name=''):
+    np.testing.assert_allclose(got, ref, rtol=rtol, atol=atol * max(1.0, float(np.abs(ref).max())), err_msg=name)
+
+
+def test_config1_conv2d_module_forward_backward():
+    """Conv2d(16, 32, 3, stride 1, pad 1, bias) on x = randn(32,16,32,32), upstream grad randn, seed 0."""
+    import pytortto_amd as tt
+    tt.manual_seed(0)
+    conv = tt.nn.Conv2d(16, 32, 3, stride=1, padding=1, bias=True)
+    x = tt.randn(32, 16, 32, 32, requires_grad=True)
+    g = tt.randn(32, 32, 32, 32)
+    w, b = conv.weight.data.copy(), conv.bias.data.copy()
+    y_ref, xpad = oracle.convolution_forward(np.asarray(x.data), np.asarray(w), np.asarray(b), (1, 1), (1, 1), (1, 1), 1)
+    dx_ref, dw_ref, db_ref = oracle.convolution_backward(np.asarray(g.data), np.asarray(x.data), xpad, np.asarray(w),
+                                                         (1, 1), (1, 1), (1, 1), 1)
+    conv.cuda()
+    xd = x.cuda()
+    assert xd.grad_fn.__class__.__name__ == 'ToCopyBackward' and str(xd.device) == 'hip:0'
+    y = conv(xd)
+    assert y.grad_fn.__class__.__name__ == 'ConvolutionBackward' and y.shape == (32, 32, 32, 32)
+    with pytest.raises(TypeError, match="can't convert hip:0 device type tensor to numpy"):
+        y.detach().numpy()
+    y.backward(g.cuda())
+    _close(y.cpu().detach().numpy(), y_ref, name='y')
+    assert type(x.grad) is np.ndarray            # came back through ToCopyBackward
+    _close(x.grad, dx_ref, name='x.grad')
+    _close(conv.weight.grad.get(), dw_ref, name='weight.grad')
+    _close(conv.bias.grad.get(), db_ref, name='bias.grad')
+    sd = conv.state_dict()
+    assert type(sd['weight']) is np.ndarray
+    np.testing.assert_array_equal(sd['weight'], w)
+
+
+def test_batchnorm2d_module_train_steps_and_eval():
+    import pytortto_amd as tt
+    tt.manual_seed(1)
+    bn = tt.nn.BatchNorm2d(6, momentum=None)      # cumulative moving average
+    xs = [2 + 3 * np.random.randn(8, 6, 16, 16).astype(np.float32) for _ in range(3)]
+    rm, rv = np.zeros(6, np.float32), np.ones(6, np.float32)
+    gamma, beta = np.ones(6, np.float32), np.zeros(6, np.float32)
+    bn.cuda()
+    for step, x in enumerate(xs):
+        y_ref, _, rm, rv = oracle.batch_norm_forward(x, gamma, beta, rm, rv, True, 1.0 / (step + 1), 1e-5)
+        y = bn(tt.tensor(x).cuda())
+        _close(y.cpu().numpy(), y_ref, rtol=1e-5, atol=2e-6)
+    assert bn.num_batches_tracked.item() == 3.0
+    sd = bn.state_dict()
+    _close(sd['running_mean'], rm, rtol=1e-5, atol=1e-6)
+    _close(sd['running_var'], rv, rtol=1e-5, atol=1e-6)
+    bn.eval()
+    y_ref, _, _, _ = oracle.batch_norm_forward(xs[0], gamma, beta, rm, rv, False, None, 1e-5)
+    _close(bn(tt.tensor(xs[0]).cuda()).cpu().numpy(), y_ref, rtol=1e-5, atol=2e-6)
+    assert bn.num_batches_tracked.item() == 3.0
+
+
+def test_conv_transpose2d_module_with_output_size():
+    import pytortto_amd as tt
+    tt.manual_seed(2)
+    m = tt.nn.ConvTranspose2d(8, 6, 3, stride=2, padding=1, groups=2)
+    x = tt.randn(3, 8, 5, 5, requires_grad=True)
+    w, b = np.asarray(m.weight.data).copy(), np.asarray(m.bias.data).copy()
+    y_ref = oracle.transposed_convolution_forward(np.asarray(x.data), w, b, (2, 2), (1, 1), (1, 1), (1, 1), 2)
+    g = np.random.randn(*y_ref.shape).astype(np.float32)
+    dx_ref, dw_ref, db_ref = oracle.transposed_convolution_backward(g, np.asarray(x.data), w, (2, 2), (1, 1), (1, 1), 2)
+    m.cuda()
+    y = m(x.cuda(), output_size=(10, 10))
+    assert y.shape == (3, 6, 10, 10) and y.grad_fn.__class__.__name__ == 'TransposedConvolutionBackward'
+    y.backward(tt.tensor(g).cuda())
+    _close(y.cpu().detach().numpy(), y_ref)
+    _close(x.grad, dx_ref)
+    _close(m.weight.grad.get(), dw_ref)
+    _close(m.bias.grad.get(), db_ref)
+
+
+def test_preact_block_on_device_matches_oracle_composition():
+    """BN-ReLU-conv3x3(s2)-BN-ReLU-conv3x3 plus a 1x1 stride-2 shortcut on the raw block input:
+    the whole block runs on the device (residual add and gradient accumulation included)."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    tt.manual_seed(4)
+    bn1, conv1 = nn.BatchNorm2d(8), nn.Conv2d(8, 16, 3, stride=2, padding=1, bias=False)
+    bn2, conv2 = nn.BatchNorm2d(16), nn.Conv2d(16, 16, 3, stride=1, padding=1, bias=False)
+    short = nn.Conv2d(8, 16, 1, stride=2, bias=False)
+    x = (1 + 2 * np.random.randn(6, 8, 12, 12)).astype(np.float32)
+    g = np.random.randn(6, 16, 6, 6).astype(np.float32)
+    w1, w2, ws = (np.asarray(m.weight.data).copy() for m in (conv1, conv2, short))
+    one8, zero8, one16, zero16 = np.ones(8, np.float32), np.zeros(8, np.float32), np.ones(16, np.float32), np.zeros(16, np.float32)
+
+    # oracle composition
+    a1, s1, _, _ = oracle.batch_norm_forward(x, one8, zero8, None, None, True, 0.1, 1e-5)
+    r1 = np.maximum(a1, 0)
+    c1, r1pad = oracle.convolution_forward(r1, w1, None, (2, 2), (1, 1), (1, 1), 1)
+    a2, s2, _, _ = oracle.batch_norm_forward(c1, one16, zero16, None, None, True, 0.1, 1e-5)
+    r2 = np.maximum(a2, 0)
+    c2, r2pad = oracle.convolution_forward(r2, w2, None, (1, 1), (1, 1), (1, 1), 1)
+    sc, xpad = oracle.convolution_forward(x, ws, None, (2, 2), (0, 0), (1, 1), 1)
+    out_ref = c2 + sc
+    d_r2, dw2_ref, _ = oracle.convolution_backward(g, r2, r2pad, w2, (1, 1), (1, 1), (1, 1), 1, need=(True, True, False))
+    d_c1, dg2_ref, db2_ref = oracle.batch_norm_backward(d_r2 * (r2 > 0), c1, one16, s2)
+    d_r1, dw1_ref, _ = oracle.convolution_backward(d_c1, r1, r1pad, w1, (2, 2), (1, 1), (1, 1), 1, need=(True, True, False))
+    dx_main, dg1_ref, db1_ref = oracle.batch_norm_backward(d_r1 * (r1 > 0), x, one8, s1)
+    dx_short, dws_ref, _ = oracle.convolution_backward(g, x, xpad, ws, (2, 2), (0, 0), (1, 1), 1, need=(True, True, False))
+    dx_ref = dx_main + dx_short
+
+    for m in (bn1, conv1, bn2, conv2, short):
+        m.cuda()
+    relu = nn.ReLU()
+    xt = tt.tensor(x, requires_grad=True)
+    xd = xt.cuda()
+    out = conv2(relu(bn2(conv1(relu(bn1(xd)))))) + short(xd)
+    out.backward(tt.tensor(g).cuda())
+    _close(out.cpu().detach().numpy(), out_ref, name='out')
+    _close(xt.grad, dx_ref, atol=2e-5, name='dx')
+    _close(conv1.weight.grad.get(), dw1_ref, atol=2e-5, name='dw1')
+    _close(conv2.weight.grad.get(), dw2_ref, atol=2e-5, name='dw2')
+    _close(short.weight.grad.get(), dws_ref, atol=2e-5, name='dws')
+    _close(bn1.weight.grad.get(), dg1_ref, atol=2e-5, name='dgamma1')
+    _close(bn2.bias.grad.get(), db2_ref, atol=2e-5, name='dbeta2')
+
+
+def test_unbatched_input_and_mixed_device_error():
+    import pytortto_amd as tt
+    tt.manual_seed(5)
+    conv = tt.nn.Conv2d(3, 4, 3, padding=1)
+    x = tt.randn(3, 6, 6)
+    w, b = np.asarray(conv.weight.data).copy(), np.asarray(conv.bias.data).copy()
+    y_ref, _ = oracle.convolution_forward(np.asarray(x.data)[None], w, b, (1, 1), (1, 1), (1, 1), 1)
+    with pytest.raises(RuntimeError, match='Input type \\(hiparray\\) and weight type \\(nparray\\) should be the same'):
+        conv(x.cuda())
+    conv.cuda()
+    y = conv(x.cuda())
+    assert y.shape == (4, 6, 6)
+    _close(y.cpu().numpy(), y_ref[0])
+
+
+def test_device_memory_is_pooled_and_released():
+    import ctypes
+    import pytortto_amd as tt
+    from pytortto_amd import _hip
+    from pytortto_amd.xparray import hiparray
+    used, pooled, ws = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    a = hiparray(np.ones((256, 256), np.float32))
+    _hip.call('tt_mem_stats', ctypes.byref(used), ctypes.byref(pooled), ctypes.byref(ws))
+    before = used.value
+    ptr = a.ptr
+    del a
+    _hip.call('tt_mem_stats', ctypes.byref(used), ctypes.byref(pooled), ctypes.byref(ws))
+    assert used.value == before - 256 * 256 * 4
+    b = hiparray(np.zeros((256, 256), np.float32))
+    assert b.ptr == ptr                       # same size class: the pooled block is reused
+    _hip.call('tt_empty_cache')

@@ -1,0 +1,163 @@
+"""CPU tests of the host-side mirror of tortto's API (no GPU, no compute through the C ABI)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+import pytortto_amd as tt
+from pytortto_amd import nn
+from pytortto_amd.build import LIB_PATH
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, 'include', 'tortto_hip.h')).read()
+    declared = set(re.findall(r'\b(tt_[a-z0-9_]+)\s*\(', header))
+    assert len(declared) >= 25
+    assert os.path.exists(LIB_PATH), 'libtortto_hip.so has not been built (python -m pytortto_amd.build)'
+    lib = ctypes.CDLL(LIB_PATH)
+    missing = [name for name in sorted(declared) if not hasattr(lib, name)]
+    assert not missing, f'symbols declared in include/tortto_hip.h but not exported: {missing}'
+    from pytortto_amd import _hip
+    assert declared == set(_hip.PROTOTYPES) | {'tt_last_error'}
+    _hip.load_library()     # attaches every prototype; makes no GPU call
+
+
+def test_seeded_conv2d_parameters_match_reference_draw_order():
+    tt.manual_seed(0)
+    conv = nn.Conv2d(16, 32, 3, stride=1, padding=1, bias=True)
+    x = tt.randn(2, 3)
+    np.random.seed(0)
+    w, b = oracle.conv_parameters(16, 32, (3, 3))
+    np.testing.assert_array_equal(conv.weight.data, w)
+    np.testing.assert_array_equal(conv.bias.data, b)
+    np.testing.assert_array_equal(x.data, np.random.randn(2, 3).astype(np.float32))
+    assert conv.weight.requires_grad and conv.weight.is_leaf and conv.weight.dtype == np.float32
+
+
+def test_conv_transpose_weight_layout_and_output_padding():
+    tt.manual_seed(1)
+    m = nn.ConvTranspose2d(8, 6, 3, stride=2, padding=1, groups=2)
+    assert m.weight.shape == (8, 3, 3, 3) and m.bias.shape == (6,)
+    x = tt.zeros(1, 8, 5, 5)
+    assert list(m._output_padding(x, None, m.stride, m.padding, m.kernel_size, m.dilation)) == [0]
+    assert m._output_padding(x, (10, 10), m.stride, m.padding, m.kernel_size, m.dilation) == [1, 1]
+    assert m._output_padding(x, (1, 6, 9, 10), m.stride, m.padding, m.kernel_size, m.dilation) == [0, 1]
+    with pytest.raises(ValueError, match='requested an output size'):
+        m._output_padding(x, (12, 12), m.stride, m.padding, m.kernel_size, m.dilation)
+    with pytest.raises(ValueError, match='Only "zeros" padding mode'):
+        nn.ConvTranspose2d(4, 4, 3, padding_mode='reflect')
+
+
+def test_constructor_errors():
+    with pytest.raises(ValueError, match='in_channels must be divisible by groups'):
+        nn.Conv2d(3, 4, 3, groups=2)
+    with pytest.raises(ValueError, match='out_channels must be divisible by groups'):
+        nn.Conv2d(4, 3, 3, groups=2)
+    with pytest.raises(ValueError, match='padding_mode must be one of'):
+        nn.Conv2d(4, 4, 3, padding_mode='circular')
+
+
+def test_host_tensors_are_refused_by_the_hot_path():
+    conv = nn.Conv2d(2, 2, 1)
+    with pytest.raises(RuntimeError, match='device \\(HIP\\) path only'):
+        conv(tt.randn(1, 2, 4, 4))
+    bn = nn.BatchNorm2d(2)
+    with pytest.raises(RuntimeError, match='device \\(HIP\\) path only'):
+        bn(tt.randn(2, 2, 4, 4))
+    with pytest.raises(ValueError, match='expected 4D input'):
+        bn(tt.randn(2, 2, 4))
+    with pytest.raises(RuntimeError, match='Expected 3D \\(unbatched\\) or 4D \\(batched\\) input to conv2d'):
+        conv(tt.randn(1, 1, 2, 4, 4))
+    with pytest.raises(RuntimeError, match='expected input'):
+        conv(tt.randn(1, 3, 4, 4))
+
+
+def test_batchnorm_module_state():
+    bn = nn.BatchNorm2d(5)
+    sd = bn.state_dict()
+    assert list(sd) == ['weight', 'bias', 'running_mean', 'running_var', 'num_batches_tracked']
+    assert sd['num_batches_tracked'].dtype == np.float32 and sd['num_batches_tracked'].shape == ()
+    np.testing.assert_array_equal(sd['running_var'], np.ones(5, np.float32))
+    assert all(type(v) is np.ndarray for v in sd.values())
+    bn2 = nn.BatchNorm2d(5, affine=False, track_running_stats=False)
+    assert bn2.weight is None and bn2.running_mean is None and list(bn2.state_dict()) == []
+
+
+def test_state_dict_round_trip_and_errors():
+    tt.manual_seed(3)
+    a = nn.Sequential(nn.Conv2d(2, 3, 3), nn.BatchNorm2d(3), nn.ReLU())
+    b = nn.Sequential(nn.Conv2d(2, 3, 3), nn.BatchNorm2d(3), nn.ReLU())
+    assert not np.array_equal(a[0].weight.data, b[0].weight.data)
+    res = b.load_state_dict(a.state_dict())
+    assert repr(res) == '<All keys matched successfully>'
+    np.testing.assert_array_equal(a[0].weight.data, b[0].weight.data)
+    bad = a.state_dict()
+    bad.pop('1.running_mean')
+    bad['extra'] = np.zeros(1)
+    with pytest.raises(RuntimeError, match='Missing key\\(s\\).*\n.*Unexpected key'):
+        b.load_state_dict(bad)
+    wrong = a.state_dict()
+    wrong['0.weight'] = np.zeros((3, 2, 1, 1), np.float32)
+    with pytest.raises(RuntimeError, match='size mismatch for 0.weight'):
+        b.load_state_dict(wrong)
+
+
+def test_module_registry_and_repr():
+    net = nn.Sequential(nn.Conv2d(3, 8, 3, padding=1, bias=False), nn.BatchNorm2d(8), nn.ReLU(inplace=True))
+    names = [n for n, _ in net.named_parameters()]
+    assert names == ['0.weight', '1.weight', '1.bias']
+    assert len(list(net.modules())) == 4 and len(net) == 3
+    assert 'Conv2d(3, 8, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), bias=False)' in repr(net)
+    net.eval()
+    assert not net[1].training
+    net.train()
+    assert net[1].training
+    with pytest.raises(KeyError):
+        net.register_buffer('a.b', None)
+    with pytest.raises(TypeError):
+        net.register_parameter('p', tt.zeros(1))
+
+
+def test_autograd_engine_on_host_add_relu():
+    """Engine semantics the path relies on: AccumulateGrad on leaves, gradient accumulation when
+    a tensor feeds two consumers (residual shortcut), grad_fn naming, cleared nodes."""
+    x = tt.tensor(np.array([-1.0, 2.0, 3.0], np.float32), requires_grad=True)
+    r = tt.nn.functional.relu(x)
+    y = r + x                     # x is used twice
+    assert y.grad_fn.__class__.__name__ == 'AddBackward' and r.grad_fn.__class__.__name__ == 'ReluBackward'
+    y.backward(tt.tensor(np.array([1.0, 10.0, 100.0], np.float32)))
+    np.testing.assert_array_equal(x.grad, np.array([1.0, 20.0, 200.0], np.float32))
+    assert type(x.grad) is np.ndarray
+    y2 = tt.nn.functional.relu(x)
+    y2.backward(tt.tensor(np.ones(3, np.float32)))
+    np.testing.assert_array_equal(x.grad, np.array([1.0, 21.0, 201.0], np.float32))   # accumulates
+    with tt.no_grad():
+        z = tt.nn.functional.relu(x)
+    assert z.grad_fn is None and not z.requires_grad
+    with pytest.raises(RuntimeError, match='does not require grad'):
+        z.backward()
+
+
+def test_inplace_version_check():
+    x = tt.tensor(np.array([1.0, -2.0], np.float32), requires_grad=True)
+    with pytest.raises(RuntimeError, match='leaf Variable that requires grad'):
+        tt.nn.functional.relu(x, inplace=True)
+    a = x + x
+    b = tt.nn.functional.relu(a)          # saves its output
+    tt.nn.functional.relu(b, inplace=True)  # bumps b's version
+    with pytest.raises(RuntimeError, match='modified by an inplace operation'):
+        b.backward(tt.tensor(np.ones(2, np.float32)))
+
+
+def test_cpu_copy_is_a_no_op_on_host_and_numpy_rules():
+    x = tt.randn(2, 2)
+    assert x.cpu() is x and x.device == 'cpu'
+    assert x.numpy() is x.data
+    x.requires_grad_(True)
+    with pytest.raises(RuntimeError, match="Can't call numpy\\(\\) on Tensor that requires grad"):
+        x.numpy()
