@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""Benchmark of the convolution / BatchNorm hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  Primary metric: fp32 conv fwd+dgrad+wgrad TFLOP/s over the 53
+convolutions of ResNet-50 at batch 64, 224x224 (one "step" = one pass over all of them, inputs
+resident in HBM, synthetic N(0,1) data, Kaiming-uniform weights).  Secondary (same line, key
+"bn"): BatchNorm2d training fwd+bwd GB/s at [64,256,56,56] and [128,64,112,112].
+
+Timing: W warm-up steps, then exactly K steps between stream synchronisations (HIP events on
+the library's stream give ms_per_step; the wall clock around the same region is reported
+too).  A second pass of K steps runs with the library's per-kernel event brackets switched on
+and yields the average launch duration of each kernel for the roofline objects; event records
+between kernels cost a few microseconds each, which is why they are not part of the first pass.
+The CPU baseline (NumPy restatement of the reference's CPU path, ``oracle/``) is timed on a
+bounded sample of the same workloads on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+# ResNet-50 convolutions at 224x224: (C_in, H_in, C_out, kernel, stride, pad, occurrences)
+RESNET50_CONVS = [
+    (3, 224, 64, 7, 2, 3, 1),
+    (64, 56, 256, 1, 1, 0, 4), (64, 56, 64, 1, 1, 0, 1), (64, 56, 64, 3, 1, 1, 3), (256, 56, 64, 1, 1, 0, 2),
+    (256, 56, 512, 1, 2, 0, 1), (256, 56, 128, 1, 1, 0, 1), (128, 56, 128, 3, 2, 1, 1),
+    (128, 28, 512, 1, 1, 0, 4), (512, 28, 128, 1, 1, 0, 3), (128, 28, 128, 3, 1, 1, 3),
+    (512, 28, 1024, 1, 2, 0, 1), (512, 28, 256, 1, 1, 0, 1), (256, 28, 256, 3, 2, 1, 1),
+    (256, 14, 1024, 1, 1, 0, 6), (1024, 14, 256, 1, 1, 0, 5), (256, 14, 256, 3, 1, 1, 5),
+    (1024, 14, 2048, 1, 2, 0, 1), (1024, 14, 512, 1, 1, 0, 1), (512, 14, 512, 3, 2, 1, 1),
+    (512, 7, 2048, 1, 1, 0, 3), (2048, 7, 512, 1, 1, 0, 2), (512, 7, 512, 3, 1, 1, 2),
+]
+BATCH = 64
+BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
+
+
+def conv_flops(n, c, h, k, r, s, p):
+    q = (h + 2 * p - r) // s + 1
+    return 2.0 * n * k * c * r * r * q * q, q
+
+
+class ConvLayer:
+    """Device buffers of one convolution shape and the three C-ABI calls on them."""
+
+    def __init__(self, spec, batch, rng):
+        from pytortto_amd.xparray import hiparray
+        c, h, k, r, s, p, count = spec
+        self.spec, self.count, self.batch = spec, count, batch
+        self.flops, q = conv_flops(batch, c, h, k, r, s, p)
+        bound = 1.0 / np.sqrt(c * r * r)
+        self.x = hiparray(rng.standard_normal((batch, c, h, h), dtype=np.float32))
+        self.w = hiparray(rng.uniform(-bound, bound, (k, c, r, r)).astype(np.float32))
+        self.dy = hiparray(rng.standard_normal((batch, k, q, q), dtype=np.float32))
+        self.y = hiparray.empty((batch, k, q, q))
+        self.dx = hiparray.empty((batch, c, h, h))
+        self.dw = hiparray.empty((k, c, r, r))
+        self.args = (batch, c, h, h, k, r, r, s, s, p, p, 1, 1, 1)
+        self.q = q
+
+    def run(self, call):
+        a = self.args
+        call('tt_conv2d_fwd_f32', self.x.ptr, self.w.ptr, None, self.y.ptr, *a)
+        call('tt_conv2d_dgrad_f32', self.dy.ptr, self.w.ptr, None, self.dx.ptr, *a, self.q, self.q)
+        call('tt_conv2d_wgrad_f32', self.x.ptr, self.dy.ptr, self.dw.ptr, *a, self.q, self.q)
+
+
+class BnLayer:
+    def __init__(self, shape, rng):
+        from pytortto_amd.xparray import hiparray
+        n, c, h, w = shape
+        self.shape = shape
+        self.bytes = 4.0 * n * c * h * w
+        self.x = hiparray((2 + 3 * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32))
+        self.dy = hiparray(rng.standard_normal(shape, dtype=np.float32))
+        self.gamma = hiparray(rng.uniform(0.5, 1.5, c).astype(np.float32))
+        self.beta = hiparray((0.1 * rng.standard_normal(c)).astype(np.float32))
+        self.rm, self.rv = hiparray(np.zeros(c, np.float32)), hiparray(np.ones(c, np.float32))
+        self.y, self.dx = hiparray.empty(shape), hiparray.empty(shape)
+        self.mean, self.var, self.sd = (hiparray.empty((c,)) for _ in range(3))
+        self.dg, self.db = hiparray.empty((c,)), hiparray.empty((c,))
+        self.dims = (n, c, h * w)
+
+    def run(self, call):
+        call('tt_bn_fwd_train_f32', self.x.ptr, self.gamma.ptr, self.beta.ptr, self.y.ptr, self.mean.ptr,
+             self.var.ptr, self.sd.ptr, self.rm.ptr, self.rv.ptr, self.rm.ptr, self.rv.ptr, 0.1, 1e-5, *self.dims)
+        call('tt_bn_bwd_f32', self.x.ptr, self.dy.ptr, self.gamma.ptr, self.mean.ptr, self.var.ptr, self.sd.ptr,
+             self.dx.ptr, self.dg.ptr, self.db.ptr, *self.dims)
+
+
+def timed_steps(hip, step, steps, warmup):
+    """(ms per step from HIP events on the library stream, wall-clock ms per step)."""
+    for _ in range(warmup):
+        step()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    e0 = hip.Event().record()
+    for _ in range(steps):
+        step()
+    e1 = hip.Event().record()
+    ms = e0.elapsed_ms(e1)
+    hip.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return ms / steps, wall / steps
+
+
+def profiled_steps(hip, step, steps):
+    hip.profile_enable(True)
+    for _ in range(steps):
+        step()
+    prof = hip.profile_read()
+    hip.profile_enable(False)
+    return prof
+
+
+def cpu_threads():
+    try:
+        from threadpoolctl import threadpool_info
+        blas = [p for p in threadpool_info() if p.get('user_api') == 'blas']
+        if blas:
+            return max(p['num_threads'] for p in blas)
+    except Exception:
+        pass
+    return len(os.sched_getaffinity(0))
+
+
+def cpu_baseline_conv(batch):
+    """Oracle fwd + dgrad + wgrad, once per unique ResNet-50 shape, at a reduced batch."""
+    import oracle
+    rng = np.random.default_rng(0)
+    flops = 0.0
+    seconds = 0.0
+    for c, h, k, r, s, p, _count in RESNET50_CONVS:
+        f, q = conv_flops(batch, c, h, k, r, s, p)
+        x = rng.standard_normal((batch, c, h, h), dtype=np.float32)
+        w = rng.standard_normal((k, c, r, r), dtype=np.float32)
+        dy = rng.standard_normal((batch, k, q, q), dtype=np.float32)
+        t0 = time.perf_counter()
+        _, xpad = oracle.convolution_forward(x, w, None, (s, s), (p, p), (1, 1), 1)
+        oracle.convolution_backward(dy, x, xpad, w, (s, s), (p, p), (1, 1), 1, need=(True, True, False))
+        seconds += time.perf_counter() - t0
+        flops += 3 * f
+    return flops, seconds
+
+
+def cpu_baseline_bn(batch_div):
+    import oracle
+    rng = np.random.default_rng(0)
+    nbytes = 0.0
+    seconds = 0.0
+    for n, c, h, w in BN_SHAPES:
+        shape = (max(1, n // batch_div), c, h, w)
+        x = (2 + 3 * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+        dy = rng.standard_normal(shape, dtype=np.float32)
+        gamma = rng.uniform(0.5, 1.5, c).astype(np.float32)
+        beta = np.zeros(c, np.float32)
+        rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+        t0 = time.perf_counter()
+        _, saved, _, _ = oracle.batch_norm_forward(x, gamma, beta, rm, rv, True, 0.1, 1e-5)
+        oracle.batch_norm_backward(dy, x, gamma, saved)
+        seconds += time.perf_counter() - t0
+        nbytes += 8 * x.nbytes
+    return nbytes, seconds
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=10)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the host-side oracle timing')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this path runs on exactly one GPU (asked for --gpus {args.gpus}); '
+              f'nothing in it is sharded, see DESIGN.md for how it would be', file=sys.stderr)
+        sys.exit(2)
+
+    from pytortto_amd import _hip
+    from pytortto_amd._paths import LIB_PATH
+    if not os.path.exists(LIB_PATH):
+        from pytortto_amd.build import build_library
+        build_library()
+    info = _hip.device_info()
+    call = _hip.call
+    rng = np.random.default_rng(0)
+
+    # ---- convolution: ResNet-50, batch 64 ------------------------------------------------------
+    layers = [ConvLayer(spec, BATCH, rng) for spec in RESNET50_CONVS]
+    flops_per_pass = sum(l.flops * l.count for l in layers)
+    assert abs(flops_per_pass / 1e9 - 523.15) < 0.05, flops_per_pass
+
+    def conv_step():
+        for l in layers:
+            for _ in range(l.count):
+                l.run(call)
+
+    conv_ms, conv_wall_ms = timed_steps(_hip, conv_step, args.steps, args.warmup)
+    conv_tflops = 3 * flops_per_pass / (conv_ms * 1e-3) / 1e12
+    prof = profiled_steps(_hip, conv_step, args.steps)
+    # dominant kernel: igemm_f32 (forward and input-gradient launches); algorithmic flops per
+    # launch = 2*N*K*C*R*S*P*Q of the layer, summed over the launches of one step
+    n_fwd, ms_fwd = prof['conv_igemm_fwd']
+    n_dg, ms_dg = prof['conv_igemm_dgrad']
+    igemm_flops = 2 * flops_per_pass * args.steps
+    igemm_tflops = igemm_flops / ((ms_fwd + ms_dg) * 1e-3) / 1e12
+    n_wg, ms_wg = prof['conv_wgrad']
+    wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
+    kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
+    del layers
+    call('tt_empty_cache')
+
+    # ---- BatchNorm2d training fwd+bwd -----------------------------------------------------------
+    bns = [BnLayer(s, rng) for s in BN_SHAPES]
+    bn_bytes = sum(8 * b.bytes for b in bns)
+
+    def bn_step():
+        for b in bns:
+            b.run(call)
+
+    bn_ms, bn_wall_ms = timed_steps(_hip, bn_step, args.steps, args.warmup)
+    bn_gbs = bn_bytes / (bn_ms * 1e-3) / 1e9
+    per_shape = {}
+    for b in bns:
+        ms, _ = timed_steps(_hip, lambda: b.run(call), args.steps, 1)
+        per_shape['x'.join(map(str, b.shape))] = round(8 * b.bytes / (ms * 1e-3) / 1e9, 1)
+    bprof = profiled_steps(_hip, bn_step, args.steps)
+    bn_kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in bprof.items() if v[0]}
+    # dominant kernel: bn_bwd_apply (reads x, dy, writes dx: 3*S algorithmic bytes per launch)
+    n_ba, ms_ba = bprof['bn_bwd_apply']
+    bwd_apply_gbs = sum(3 * b.bytes for b in bns) * args.steps / (ms_ba * 1e-3) / 1e9
+    del bns
+    call('tt_empty_cache')
+
+    # ---- CPU baseline (oracle on the host cores) -------------------------------------------------
+    cpu_conv = cpu_bn = None
+    if not args.no_cpu_baseline:
+        cores = cpu_threads()
+        cbatch = 8
+        f, sec = cpu_baseline_conv(cbatch)
+        cpu_conv = {'value': round(f / sec / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
+                    'sample': f'oracle fwd+dgrad+wgrad once over the 23 unique ResNet-50 conv shapes at batch '
+                              f'{cbatch} ({f / 1e9:.0f} GFLOP counted, {sec:.1f} s)'}
+        nb, sec = cpu_baseline_bn(2)
+        cpu_bn = {'value': round(nb / sec / 1e9, 3), 'unit': 'GB/s', 'cores': cores, 'kind': 'port',
+                  'sample': f'oracle BatchNorm fwd+bwd at both shapes with batch/2 ({nb / 1e9:.2f} GB counted, '
+                            f'{sec:.1f} s)'}
+
+    out = {
+        'metric': 'conv fwd+bwd TFLOP/s (% fp32 MFMA peak); BatchNorm2d fwd+bwd GB/s (% HBM)',
+        'value': round(conv_tflops, 2), 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(conv_ms, 3), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'ResNet-50 convolutions (53 layers, 23 unique shapes), batch 64, 3x224x224: '
+                               'fwd + dgrad + wgrad of every layer per step, 1569.5 GFLOP',
+                   'global_batch': BATCH, 'device': info['name'].strip(), 'compute_units': info['compute_units']},
+        'pct_of_peak': round(100 * conv_tflops / PEAK_FP32_MFMA_TFLOPS, 1),
+        'wall_ms_per_step': round(conv_wall_ms, 3),
+        'roofline': {'bound': 'mfma', 'kernel': 'igemm_f32 (Conv2d forward + input gradient)',
+                     'achieved': round(igemm_tflops, 2), 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': round(igemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4), 'traffic': None,
+                     'launches_per_step': (n_fwd + n_dg) // args.steps,
+                     'avg_launch_ms': round((ms_fwd + ms_dg) / max(1, n_fwd + n_dg), 5)},
+        'kernels_ms_per_step': kernel_ms,
+        'wgrad_tflops': round(wgrad_tflops, 2),
+        'cpu_baseline': cpu_conv,
+        'bn': {'metric': 'BatchNorm2d training fwd+bwd GB/s', 'value': round(bn_gbs, 1), 'unit': 'GB/s',
+               'ms_per_step': round(bn_ms, 4), 'wall_ms_per_step': round(bn_wall_ms, 4),
+               'pct_of_peak': round(100 * bn_gbs / PEAK_HBM_GBS, 1),
+               'config': {'workload': 'BatchNorm2d train fwd+bwd fp32 NCHW at [64,256,56,56] and [128,64,112,112], '
+                                      'x ~ N(2,3), 8*S algorithmic bytes per shape'},
+               'per_shape_gbs': per_shape,
+               'roofline': {'bound': 'hbm', 'kernel': 'bn_bwd_apply (reads x, dy; writes dx)',
+                            'achieved': round(bwd_apply_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                            'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4), 'traffic': None,
+                            'avg_launch_ms': round(ms_ba / max(1, n_ba), 5)},
+               'kernels_ms_per_step': bn_kernel_ms,
+               'cpu_baseline': cpu_bn},
+    }
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

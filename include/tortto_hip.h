@@ -50,6 +50,26 @@ int tt_event_record(void* event);
 int tt_event_elapsed_ms(void* start, void* stop, float* ms);   /* waits for `stop` */
 int tt_event_destroy(void* event);
 
+/* Per-kernel timing (no counterpart in the reference).  While enabled, the library brackets
+ * each launch of its main kernels with HIP events on its stream; tt_profile_read() waits for
+ * the stream and returns the number of launches and their summed duration since
+ * tt_profile_enable(1).  Event records between kernels cost a few microseconds each, so
+ * whole-job throughput is measured with profiling off. */
+enum {
+  TT_PROF_CONV_IGEMM_FWD = 0,   /* igemm_f32 launched by tt_conv2d_fwd_f32 */
+  TT_PROF_CONV_IGEMM_DGRAD = 1, /* igemm_f32 launched by tt_conv2d_dgrad_f32 (all parity classes) */
+  TT_PROF_CONV_WGRAD = 2,       /* wgrad_f32 */
+  TT_PROF_CONV_WGRAD_REDUCE = 3,
+  TT_PROF_CONV_PREP = 4,        /* weight repack + reduction-index table kernels */
+  TT_PROF_BN_FWD_REDUCE = 5,
+  TT_PROF_BN_FWD_APPLY = 6,
+  TT_PROF_BN_BWD_REDUCE = 7,
+  TT_PROF_BN_BWD_APPLY = 8,
+  TT_PROF_COUNT = 9
+};
+int tt_profile_enable(int on);
+int tt_profile_read(int kernel_id, long long* launches, double* total_ms);
+
 /* ---- convolution ------------------------------------------------------------------------- */
 
 /* y[N,K,P,Q] = conv(x[N,C,H,W], w[K,C/groups,R,S]) (+ bias[K] if not NULL).

@@ -8,7 +8,7 @@ import ctypes
 import os
 from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
 
-from .build import LIB_PATH
+from ._paths import LIB_PATH
 
 _P = c_void_p
 _I = c_int
@@ -30,6 +30,8 @@ PROTOTYPES = {
     'tt_event_record': [_P],
     'tt_event_elapsed_ms': [_P, _P, POINTER(c_float)],
     'tt_event_destroy': [_P],
+    'tt_profile_enable': [_I],
+    'tt_profile_read': [_I, POINTER(ctypes.c_longlong), POINTER(c_double)],
     'tt_conv2d_fwd_f32': [_P, _P, _P, _P] + [_I] * 14,
     'tt_conv2d_dgrad_f32': [_P, _P, _P, _P] + [_I] * 16,
     'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
@@ -102,6 +104,26 @@ def device_info():
     call('tt_device_info', name, 256, ctypes.byref(cus), ctypes.byref(khz), ctypes.byref(lds), ctypes.byref(mem))
     return {'name': name.value.decode(), 'compute_units': cus.value, 'clock_khz': khz.value,
             'lds_bytes_per_block': lds.value, 'total_mem_bytes': mem.value}
+
+
+PROF_KERNELS = {
+    'conv_igemm_fwd': 0, 'conv_igemm_dgrad': 1, 'conv_wgrad': 2, 'conv_wgrad_reduce': 3, 'conv_prep': 4,
+    'bn_fwd_reduce': 5, 'bn_fwd_apply': 6, 'bn_bwd_reduce': 7, 'bn_bwd_apply': 8,
+}
+
+
+def profile_enable(on=True):
+    call('tt_profile_enable', 1 if on else 0)
+
+
+def profile_read():
+    """{kernel name: (launches, total milliseconds)} since ``profile_enable(True)``."""
+    out = {}
+    for name, kid in PROF_KERNELS.items():
+        n, ms = ctypes.c_longlong(), c_double()
+        call('tt_profile_read', kid, ctypes.byref(n), ctypes.byref(ms))
+        out[name] = (n.value, ms.value)
+    return out
 
 
 def synchronize():

@@ -10,11 +10,7 @@ import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(HERE, 'csrc')
-OBJ_DIR = os.path.join(CSRC, 'build')
-LIB_DIR = os.path.join(HERE, 'lib')
-LIB_PATH = os.path.join(LIB_DIR, 'libtortto_hip.so')
+from pytortto_amd._paths import CSRC, LIB_DIR, LIB_PATH, OBJ_DIR
 
 ARCH = 'gfx950'
 # packed-fp32 instructions are switched off for the device code of every kernel in this library

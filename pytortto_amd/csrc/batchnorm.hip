@@ -455,7 +455,10 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   void* ws;
   if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
   dim3 grid(g.splits, C);
-  launch_reduce<0>(mode, grid, x, x, nullptr, (double2*)ws, g);
+  {
+    tt::ProfScope prof(TT_PROF_BN_FWD_REDUCE);
+    launch_reduce<0>(mode, grid, x, x, nullptr, (double2*)ws, g);
+  }
   TT_LAUNCH_CHECK();
   FwdArgs a{};
   a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
@@ -469,9 +472,12 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   a.unbias = (float)((double)m / (double)(m - 1));
   a.eps = (float)eps;
   hipStream_t st = tt::stream();
-  if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  {
+    tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
+    if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  }
   TT_LAUNCH_CHECK();
   return 0;
 }
@@ -493,9 +499,12 @@ int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, fl
   a.given_mean = mean; a.given_var = var;
   a.eps = (float)eps;
   hipStream_t st = tt::stream();
-  if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  {
+    tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
+    if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  }
   TT_LAUNCH_CHECK();
   return 0;
 }
@@ -513,13 +522,19 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const flo
   void* ws;
   if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
   dim3 grid(g.splits, C);
-  launch_reduce<1>(mode, grid, x, dy, save_mean, (double2*)ws, g);
+  {
+    tt::ProfScope prof(TT_PROF_BN_BWD_REDUCE);
+    launch_reduce<1>(mode, grid, x, dy, save_mean, (double2*)ws, g);
+  }
   TT_LAUNCH_CHECK();
   BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws};
   hipStream_t st = tt::stream();
-  if (mode == 0) bn_bwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 1) bn_bwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
-  if (mode == 2) bn_bwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  {
+    tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
+    if (mode == 0) bn_bwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 1) bn_bwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+    if (mode == 2) bn_bwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+  }
   TT_LAUNCH_CHECK();
   return 0;
 }

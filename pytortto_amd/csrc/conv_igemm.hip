@@ -305,7 +305,8 @@ TileChoice choose_tile(int I, int M, int groups) {
   return t;
 }
 
-int launch_igemm(Igemm& p, int groups, TileChoice t) {
+int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id) {
+  tt::ProfScope prof(prof_id);
   p.tilesI = p.Ipad / t.bm;
   p.tiles = p.tilesI * ceil_div(p.M, t.bn);
   dim3 grid(p.tiles, groups);
@@ -366,11 +367,14 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   floatx4* wp = (floatx4*)ws;
   KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
   hipStream_t st = tt::stream();
-  pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ);
-  TT_LAUNCH_CHECK();
-  KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
-  build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
-  TT_LAUNCH_CHECK();
+  {
+    tt::ProfScope prof(TT_PROF_CONV_PREP);
+    pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ);
+    TT_LAUNCH_CHECK();
+    KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
+    build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
+    TT_LAUNCH_CHECK();
+  }
 
   Igemm p{};
   p.src = x; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = y;
@@ -382,7 +386,7 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   p.srcStrideN = C * H * W; p.srcStrideG = Cg * H * W;
   p.outStrideN = K * P * Q; p.outStrideG = Kg * P * Q; p.outStrideI = P * Q; p.outRow = Q;
   p.ou = 1; p.ouh = 0; p.ov = 1; p.ovw = 0;
-  return launch_igemm(p, groups, t);
+  return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD);
 }
 
 int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
@@ -431,6 +435,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
       Igemm p{};
       if (KQ > 0) {
+        tt::ProfScope prof(TT_PROF_CONV_PREP);
         PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
         pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa);
         TT_LAUNCH_CHECK();
@@ -450,7 +455,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       p.srcStrideN = K * P * Q; p.srcStrideG = Kg * P * Q;
       p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
       p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
-      if (launch_igemm(p, groups, t)) return -1;
+      if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD)) return -1;
     }
   }
   return 0;

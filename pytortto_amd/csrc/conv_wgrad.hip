@@ -254,6 +254,8 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   p.outStrideSplit = elems;
   dim3 grid(tilesI * tilesJ, groups, splits);
   hipStream_t st = tt::stream();
+  {
+  tt::ProfScope prof(TT_PROF_CONV_WGRAD);
   if (bm == 128 && bn == 128)
     wgrad_f32<2, 2, 2, 2><<<grid, kThreads, 0, st>>>(p);
   else if (bm == 64 && bn == 128)
@@ -262,8 +264,10 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
     wgrad_f32<2, 2, 2, 1><<<grid, kThreads, 0, st>>>(p);
   else
     wgrad_f32<2, 2, 1, 1><<<grid, kThreads, 0, st>>>(p);
+  }
   TT_LAUNCH_CHECK();
   if (splits > 1) {
+    tt::ProfScope prof(TT_PROF_CONV_WGRAD_REDUCE);
     wgrad_reduce<<<ceil_div((long long)elems, kThreads), kThreads, 0, st>>>(target, dw, elems, splits);
     TT_LAUNCH_CHECK();
   }

@@ -25,6 +25,16 @@ struct State {
   size_t bytes_pooled = 0;
   void* ws = nullptr;
   size_t ws_bytes = 0;
+  // per-kernel timing
+  bool profiling = false;
+  std::vector<hipEvent_t> event_pool;
+  struct Pending {
+    int id;
+    hipEvent_t start, stop;
+  };
+  std::vector<Pending> pending;
+  long long prof_launches[TT_PROF_COUNT] = {};
+  double prof_ms[TT_PROF_COUNT] = {};
 };
 
 State& S() {
@@ -89,6 +99,38 @@ int workspace(size_t bytes, void** out) {
   }
   *out = s.ws;
   return 0;
+}
+
+ProfScope::ProfScope(int kernel_id) : id(kernel_id), start(nullptr) {
+  State& s = S();
+  if (!s.profiling) return;
+  hipEvent_t e = nullptr;
+  if (!s.event_pool.empty()) {
+    e = s.event_pool.back();
+    s.event_pool.pop_back();
+  } else if (hipEventCreate(&e) != hipSuccess) {
+    return;
+  }
+  if (hipEventRecord(e, s.stream) != hipSuccess) {
+    s.event_pool.push_back(e);
+    return;
+  }
+  start = (void*)e;
+}
+
+ProfScope::~ProfScope() {
+  if (!start) return;
+  State& s = S();
+  hipEvent_t e = nullptr;
+  if (!s.event_pool.empty()) {
+    e = s.event_pool.back();
+    s.event_pool.pop_back();
+  } else if (hipEventCreate(&e) != hipSuccess) {
+    s.event_pool.push_back((hipEvent_t)start);
+    return;
+  }
+  (void)hipEventRecord(e, s.stream);
+  s.pending.push_back({id, (hipEvent_t)start, e});
 }
 
 FastDiv make_fastdiv(uint32_t d) {
@@ -234,6 +276,42 @@ int tt_memset(void* dst_dev, int byte_value, size_t bytes) {
 int tt_sync(void) {
   TT_REQUIRE_INIT();
   TT_HIP(hipStreamSynchronize(S().stream));
+  return 0;
+}
+
+int tt_profile_enable(int on) {
+  TT_REQUIRE_INIT();
+  State& s = S();
+  TT_HIP(hipStreamSynchronize(s.stream));
+  for (auto& p : s.pending) {
+    s.event_pool.push_back(p.start);
+    s.event_pool.push_back(p.stop);
+  }
+  s.pending.clear();
+  for (int i = 0; i < TT_PROF_COUNT; ++i) {
+    s.prof_launches[i] = 0;
+    s.prof_ms[i] = 0.0;
+  }
+  s.profiling = on != 0;
+  return 0;
+}
+
+int tt_profile_read(int kernel_id, long long* launches, double* total_ms) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(kernel_id >= 0 && kernel_id < TT_PROF_COUNT, "tt_profile_read: unknown kernel id %d", kernel_id);
+  State& s = S();
+  TT_HIP(hipStreamSynchronize(s.stream));
+  for (auto& p : s.pending) {
+    float ms = 0.f;
+    TT_HIP(hipEventElapsedTime(&ms, p.start, p.stop));
+    s.prof_launches[p.id] += 1;
+    s.prof_ms[p.id] += (double)ms;
+    s.event_pool.push_back(p.start);
+    s.event_pool.push_back(p.stop);
+  }
+  s.pending.clear();
+  if (launches) *launches = s.prof_launches[kernel_id];
+  if (total_ms) *total_ms = s.prof_ms[kernel_id];
   return 0;
 }
 

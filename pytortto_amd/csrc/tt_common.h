@@ -21,6 +21,14 @@ bool initialised();
 // more; work on the stream is ordered, so consecutive launches may reuse it.
 int workspace(size_t bytes, void** out);
 
+// Brackets the launches made during its lifetime with events when profiling is enabled.
+struct ProfScope {
+  explicit ProfScope(int kernel_id);
+  ~ProfScope();
+  int id;
+  void* start;
+};
+
 constexpr int kWave = 64;
 
 inline bool fits_i32(long long elems) { return elems >= 0 && elems < 2147483647LL; }

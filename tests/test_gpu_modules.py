@@ -52,14 +52,14 @@ def test_batchnorm2d_module_train_steps_and_eval():
     for step, x in enumerate(xs):
         y_ref, _, rm, rv = oracle.batch_norm_forward(x, gamma, beta, rm, rv, True, 1.0 / (step + 1), 1e-5)
         y = bn(tt.tensor(x).cuda())
-        _close(y.cpu().numpy(), y_ref, rtol=1e-5, atol=2e-6)
+        _close(y.cpu().detach().numpy(), y_ref, rtol=1e-5, atol=2e-6)
     assert bn.num_batches_tracked.item() == 3.0
     sd = bn.state_dict()
     _close(sd['running_mean'], rm, rtol=1e-5, atol=1e-6)
     _close(sd['running_var'], rv, rtol=1e-5, atol=1e-6)
     bn.eval()
     y_ref, _, _, _ = oracle.batch_norm_forward(xs[0], gamma, beta, rm, rv, False, None, 1e-5)
-    _close(bn(tt.tensor(xs[0]).cuda()).cpu().numpy(), y_ref, rtol=1e-5, atol=2e-6)
+    _close(bn(tt.tensor(xs[0]).cuda()).cpu().detach().numpy(), y_ref, rtol=1e-5, atol=2e-6)
     assert bn.num_batches_tracked.item() == 3.0
 
 
@@ -140,7 +140,7 @@ def test_unbatched_input_and_mixed_device_error():
     conv.cuda()
     y = conv(x.cuda())
     assert y.shape == (4, 6, 6)
-    _close(y.cpu().numpy(), y_ref[0])
+    _close(y.cpu().detach().numpy(), y_ref[0])
 
 
 def test_device_memory_is_pooled_and_released():
