@@ -58,9 +58,30 @@ struct Igemm {
 
 // ---- preparation kernels (tiny) --------------------------------------------------------------
 
+// k -> {offset, steps}.  k = (a*TB + b)*TC + c:  off = a*sa + b*sb + c*sc, steps (b*stepH, c*stepW).
+struct KTabArgs {
+  int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
+};
+__device__ __forceinline__ void write_ktab_entry(KEntry* __restrict__ tab, const KTabArgs& a, int k) {
+  KEntry e;
+  if (k < a.Kred) {
+    const int c = k % a.TC, t = k / a.TC;
+    const int b = t % a.TB, aa = t / a.TB;
+    e.off = aa * a.sa + b * a.sb + c * a.sc;
+    e.dhw = ((b * a.stepH) & 0xffff) | ((c * a.stepW) << 16);
+  } else {
+    e.off = 0;
+    e.dhw = (-16384) & 0xffff;   // row far above the image: never valid
+  }
+  tab[k] = e;
+}
+
 // Forward: Wp[g][kq][i][j] = w[g*I + i][4*kq + j]  (w rows are Kred = Cg*R*S long, 0 beyond).
-__global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp, int I, int Ipad, int Kred, int KQ) {
+// The first block of every k-quad also writes that quad's four table entries.
+__global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp, int I, int Ipad, int Kred, int KQ,
+                           KEntry* __restrict__ tab, KTabArgs ta) {
   const int g = blockIdx.z, kq = blockIdx.y;
+  if (blockIdx.x == 0 && g == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= Ipad) return;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -79,8 +100,10 @@ struct PackDgrad {
   int Kg, Cg, R, S, Ipad, Kred, KQ;
   int nTr, nTs, r0, rstep, s0, sstep;
 };
-__global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ wp, PackDgrad a) {
+__global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ wp, PackDgrad a,
+                             KEntry* __restrict__ tab, KTabArgs ta) {
   const int g = blockIdx.z, kq = blockIdx.y;
+  if (blockIdx.x == 0 && g == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= a.Ipad) return;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -96,26 +119,6 @@ __global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ 
     }
   }
   wp[((size_t)g * a.KQ + kq) * a.Ipad + c] = floatx4{v[0], v[1], v[2], v[3]};
-}
-
-// k -> {offset, steps}.  k = (a*TB + b)*TC + c:  off = a*sa + b*sb + c*sc, steps (b*stepH, c*stepW).
-struct KTabArgs {
-  int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
-};
-__global__ void build_ktab(KEntry* __restrict__ tab, KTabArgs a) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k >= a.Kpad) return;
-  KEntry e;
-  if (k < a.Kred) {
-    const int c = k % a.TC, t = k / a.TC;
-    const int b = t % a.TB, aa = t / a.TB;
-    e.off = aa * a.sa + b * a.sb + c * a.sc;
-    e.dhw = ((b * a.stepH) & 0xffff) | ((c * a.stepW) << 16);
-  } else {
-    e.off = 0;
-    e.dhw = (-16384) & 0xffff;   // row far above the image: never valid
-  }
-  tab[k] = e;
 }
 
 // ---- the GEMM kernel -----------------------------------------------------------------------------
@@ -167,39 +170,49 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
 
   floatx4 areg[A_ITEMS];
   floatx4 breg[B_ITEMS];
-  bool bok[B_ITEMS][4];   // applied when the values are written to LDS, after the MFMAs
+  bool bok[B_ITEMS][4];   // applied when the values are written to LDS
+  constexpr int nB = 4 * B_ITEMS;
+  intx2 tab_e[nB];        // table entries {off, dhw} of the chunk being fetched (SGPRs)
 
-  auto load_global = [&](int chunk) {
-#pragma unroll
-    for (int it = 0; it < A_ITEMS; ++it) {
-      const int kq = chunk * kBKQ + aq0 + it * (kThreads / BM);
-      areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
-    }
+  auto load_tab = [&](int chunk) {
 #pragma unroll
     for (int it = 0; it < B_ITEMS; ++it) {
       const int kq = chunk * kBKQ + bq0 + it * (kThreads / BN);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const intx2 e = ktab[kq * 4 + j];   // {off, dhw} of KEntry
-        const int ih = ih0 + (int)(short)(e.y & 0xffff);
-        const int iw = iw0 + (e.y >> 16);
-        const bool ok = (unsigned)ih < (unsigned)p.Hlim && (unsigned)iw < (unsigned)p.Wlim;
-        const uint32_t off = ok ? (uint32_t)(base + e.x) : 0u;
-        breg[it][j] = p.src[off];
-        bok[it][j] = ok;
-      }
+      for (int j = 0; j < 4; ++j) tab_e[it * 4 + j] = ktab[kq * 4 + j];
     }
   };
-  auto store_lds = [&](int buf) {
+  auto load_a_item = [&](int chunk, int it) {
+    const int kq = chunk * kBKQ + aq0 + it * (kThreads / BM);
+    areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
+  };
+  auto load_b_elem = [&](int e) {   // uses tab_e: must follow load_tab() of the same chunk
+    const intx2 t = tab_e[e];
+    const int ih = ih0 + (int)(short)(t.y & 0xffff);
+    const int iw = iw0 + (t.y >> 16);
+    const bool ok = (unsigned)ih < (unsigned)p.Hlim && (unsigned)iw < (unsigned)p.Wlim;
+    const uint32_t off = ok ? (uint32_t)(base + t.x) : 0u;
+    breg[e >> 2][e & 3] = p.src[off];
+    bok[e >> 2][e & 3] = ok;
+  };
+  auto store_a_item = [&](int buf, int it) { As[buf][aq0 + it * (kThreads / BM)][arow] = areg[it]; };
+  auto store_b_item = [&](int buf, int it) {
+    floatx4 v;
 #pragma unroll
-    for (int it = 0; it < A_ITEMS; ++it) As[buf][aq0 + it * (kThreads / BM)][arow] = areg[it];
+    for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
+    Bs[buf][bq0 + it * (kThreads / BN)][pix] = v;
+  };
+
+  // MFMA operands of one chunk: [kk][tile] float4 = four k-steps each.  Lanes 0-31 take quad
+  // 2*kk, lanes 32-63 quad 2*kk+1, so MFMA step j of half kk contracts k = 4*(2*kk + h) + j.
+  floatx4 opA[2][2][MT], opB[2][2][NT];
+  auto read_ops = [&](int set, int buf) {
 #pragma unroll
-    for (int it = 0; it < B_ITEMS; ++it)
-    {
-      floatx4 v;
+    for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
-      Bs[buf][bq0 + it * (kThreads / BN)][pix] = v;
+      for (int x = 0; x < MT; ++x) opA[set][kk][x] = As[buf][kk * 2 + h][(wm * MT + x) * 32 + l32];
+#pragma unroll
+      for (int y = 0; y < NT; ++y) opB[set][kk][y] = Bs[buf][kk * 2 + h][(wn * NT + y) * 32 + l32];
     }
   };
 
@@ -211,39 +224,81 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  // One chunk of MFMAs (operand set `set`, read from LDS buffer `set` earlier) with the work for
+  // the following chunks woven in between them, one small step per MFMA, so that it executes in
+  // the shadow of the 64-cycle matrix instructions:
+  //   slots 0..      : global loads of chunk `nchunk` (gathered elements, then weight quads)
+  //   slots T-8..    : write them to the other LDS buffer
+  //   slot  T-4      : barrier, fetch the operands of the next chunk from LDS, and start the
+  //                    scalar loads of the table entries of chunk `nnchunk`
+  // sched_barrier pins this order; the compiler otherwise sinks the loads below the MFMAs.
+  constexpr int T = 8 * MT * NT;
+  auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) {
+    if constexpr (T >= 32) {
+      constexpr int kStore = T - 8, kSync = T - 4;
+      static_assert(nB + A_ITEMS <= kStore && kStore + B_ITEMS + A_ITEMS - 1 <= kSync, "schedule does not fit");
+#pragma unroll
+      for (int s = 0; s < T; ++s) {
+        const int kk = s / (4 * MT * NT), rem = s % (4 * MT * NT);
+        const int j = rem / (MT * NT), x = (rem % (MT * NT)) / NT, y = rem % NT;
+        acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[set][kk][x][j], opB[set][kk][y][j], acc[x][y], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s < nB) load_b_elem(s);
+        else if (s < nB + A_ITEMS) load_a_item(nchunk, s - nB);
+        if (s >= kStore && s < kStore + B_ITEMS) store_b_item(set ^ 1, s - kStore);
+        else if (s >= kStore + B_ITEMS && s < kStore + B_ITEMS + A_ITEMS) store_a_item(set ^ 1, s - kStore - B_ITEMS);
+        if (s == kSync) {
+          __syncthreads();
+          read_ops(set ^ 1, set ^ 1);
+          load_tab(nnchunk);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < nB; ++e) load_b_elem(e);
+#pragma unroll
+      for (int it = 0; it < A_ITEMS; ++it) load_a_item(nchunk, it);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < T; ++s) {
+        const int kk = s / (4 * MT * NT), rem = s % (4 * MT * NT);
+        const int j = rem / (MT * NT), x = (rem % (MT * NT)) / NT, y = rem % NT;
+        acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[set][kk][x][j], opB[set][kk][y][j], acc[x][y], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int it = 0; it < B_ITEMS; ++it) store_b_item(set ^ 1, it);
+#pragma unroll
+      for (int it = 0; it < A_ITEMS; ++it) store_a_item(set ^ 1, it);
+      __syncthreads();
+      read_ops(set ^ 1, set ^ 1);
+      load_tab(nnchunk);
+    }
+  };
+
   const int chunks = p.KQ / kBKQ;
   if (chunks > 0) {
-    load_global(0);
-    store_lds(0);
+    load_tab(0);
+#pragma unroll
+    for (int e = 0; e < nB; ++e) load_b_elem(e);
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) load_a_item(0, it);
+#pragma unroll
+    for (int it = 0; it < B_ITEMS; ++it) store_b_item(0, it);
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) store_a_item(0, it);
     __syncthreads();
-  }
-  for (int c = 0; c < chunks; ++c) {
-    const int cur = c & 1;
-    // the last iteration re-fetches its own chunk (cache hit) into the idle buffer: keeping the
-    // loop body free of conditions lets the prefetch registers stay registers
-    load_global(min(c + 1, chunks - 1));
-    __builtin_amdgcn_sched_barrier(0);   // keep the prefetch ahead of the MFMAs it overlaps with
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      // lanes 0-31 take quad 2*kk, lanes 32-63 quad 2*kk+1: MFMA step j contracts k = 4*quad + j
-      floatx4 a[MT], b[NT];
-#pragma unroll
-      for (int x = 0; x < MT; ++x) a[x] = As[cur][kk * 2 + h][(wm * MT + x) * 32 + l32];
-#pragma unroll
-      for (int x = 0; x < NT; ++x) b[x] = Bs[cur][kk * 2 + h][(wn * NT + x) * 32 + l32];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int x = 0; x < MT; ++x)
-#pragma unroll
-          for (int y = 0; y < NT; ++y) {
-            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x][j], b[y][j], acc[x][y], 0, 0, 0);
-          }
-      }
+    read_ops(0, 0);
+    load_tab(min(1, chunks - 1));
+    // the last chunks re-fetch the final chunk (cache hits) instead of branching: a loop body
+    // free of conditions keeps the prefetch registers in registers
+    int c = 0;
+    for (; c + 1 < chunks; c += 2) {
+      chunk_body(0, c + 1, min(c + 2, chunks - 1));
+      chunk_body(1, min(c + 2, chunks - 1), min(c + 3, chunks - 1));
     }
-    __builtin_amdgcn_sched_barrier(0);
-    store_lds(cur ^ 1);
-    __syncthreads();
+    if (c < chunks) chunk_body(0, c, c);
   }
 
   // epilogue: accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*h + r%4, column l32
@@ -369,10 +424,8 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   hipStream_t st = tt::stream();
   {
     tt::ProfScope prof(TT_PROF_CONV_PREP);
-    pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ);
-    TT_LAUNCH_CHECK();
     KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
-    build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
+    pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
     TT_LAUNCH_CHECK();
   }
 
@@ -437,10 +490,8 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       if (KQ > 0) {
         tt::ProfScope prof(TT_PROF_CONV_PREP);
         PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
-        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa);
-        TT_LAUNCH_CHECK();
         KTabArgs ka{Kred, KQ * 4, nTr, nTs, P * Q, -eh * Q, -ew, -eh, -ew};
-        build_ktab<<<ceil_div(KQ * 4, 256), 256, 0, st>>>(tab, ka);
+        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
         TT_LAUNCH_CHECK();
         // h = u*sh + ch reads dy row (h + ph - r0*dh)/sh = u + (ch + ph - r0*dh)/sh  (exact)
         p.bh = (ch + ph - r0 * dh) / sh;   // numerator is a multiple of sh by choice of r0

@@ -183,14 +183,49 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
   }
 }
 
-// dw[e] = sum over splits of partial[s][e], added in split order in float64.
+// dw[e] = sum over splits of partial[s][e] in float64.  A block covers 64 float4 columns with
+// 4 lanes per column; lane l adds splits l, l+4, ... in order, the four lane sums are added in
+// lane order: the summation order is fixed, so the result is deterministic.
 __global__ __launch_bounds__(kThreads) void wgrad_reduce(const float* __restrict__ partial, float* __restrict__ dw,
                                                          size_t elems, int splits) {
-  const size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x;
-  if (e >= elems) return;
-  double s = 0.0;
-  for (int k = 0; k < splits; ++k) s += (double)partial[(size_t)k * elems + e];
-  dw[e] = (float)s;
+  __shared__ double lds[3][64][4];
+  const int col = threadIdx.x & 63, lane = threadIdx.x >> 6;
+  const size_t e = ((size_t)blockIdx.x * 64 + col) * 4;
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+  const bool vec = (elems & 3) == 0;   // partial rows stay 16-byte aligned
+  if (vec && e < elems) {
+#pragma unroll 2
+    for (int k = lane; k < splits; k += 4) {
+      const floatx4 v = *reinterpret_cast<const floatx4*>(partial + (size_t)k * elems + e);
+      s0 += (double)v[0]; s1 += (double)v[1]; s2 += (double)v[2]; s3 += (double)v[3];
+    }
+  } else if (e < elems) {
+    for (int k = lane; k < splits; k += 4) {
+      const float* q = partial + (size_t)k * elems + e;
+      s0 += (double)q[0];
+      if (e + 1 < elems) s1 += (double)q[1];
+      if (e + 2 < elems) s2 += (double)q[2];
+      if (e + 3 < elems) s3 += (double)q[3];
+    }
+  }
+  if (lane > 0) {
+    lds[lane - 1][col][0] = s0; lds[lane - 1][col][1] = s1; lds[lane - 1][col][2] = s2; lds[lane - 1][col][3] = s3;
+  }
+  __syncthreads();
+  if (lane == 0 && e < elems) {
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+      s0 += lds[l][col][0]; s1 += lds[l][col][1]; s2 += lds[l][col][2]; s3 += lds[l][col][3];
+    }
+    if (vec) {
+      *reinterpret_cast<floatx4*>(dw + e) = floatx4{(float)s0, (float)s1, (float)s2, (float)s3};
+    } else {
+      dw[e] = (float)s0;
+      if (e + 1 < elems) dw[e + 1] = (float)s1;
+      if (e + 2 < elems) dw[e + 2] = (float)s2;
+      if (e + 3 < elems) dw[e + 3] = (float)s3;
+    }
+  }
 }
 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
@@ -268,7 +303,7 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   TT_LAUNCH_CHECK();
   if (splits > 1) {
     tt::ProfScope prof(TT_PROF_CONV_WGRAD_REDUCE);
-    wgrad_reduce<<<ceil_div((long long)elems, kThreads), kThreads, 0, st>>>(target, dw, elems, splits);
+    wgrad_reduce<<<ceil_div((long long)elems, 256), kThreads, 0, st>>>(target, dw, elems, splits);
     TT_LAUNCH_CHECK();
   }
   return 0;
