@@ -108,32 +108,44 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_planes(const float* __rest
                                                              double2* __restrict__ partial, Geometry g) {
   __shared__ double lds[2 * kWaves];
   const int c = blockIdx.y, split = blockIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   constexpr bool kBwd = kKind == 1;
   const int hw4 = g.HW >> 2;
   const float ref = kKind == 1 ? mean[c] : (kKind == 0 ? x[(size_t)c * g.HW] : 0.f);
   const int n0 = split * g.per_block;
   const int n1 = min(g.N, n0 + g.per_block);
   double sa = 0.0, sb = 0.0;
-  for (int n = n0 + wave; n < n1; n += kWaves) {
+  // The whole block streams one plane at a time (a contiguous HW*4-byte region): batches of kU
+  // float4 loads per thread, all issued before the first is consumed; threads past the end of
+  // the plane take `ref` (a zero contribution) instead of branching out.
+  constexpr int kU = kBwd ? 2 : 4;
+  const float4 fill = make_float4(ref, ref, ref, ref);
+  for (int n = n0; n < n1; ++n) {
     const size_t off = ((size_t)n * g.C + c) * g.HW;
     const float4* __restrict__ px = reinterpret_cast<const float4*>(x + off);
     const float4* __restrict__ pg = reinterpret_cast<const float4*>(dy + (kBwd ? off : 0));
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-#pragma unroll 4
-    for (int i = lane; i < hw4; i += tt::kWave) {
-      float4 v = px[i];
-      v.x -= ref; v.y -= ref; v.z -= ref; v.w -= ref;
-      if (kBwd) {
-        const float4 gq = pg[i];
-        a.x += gq.x; a.y += gq.y; a.z += gq.z; a.w += gq.w;
-        b.x = fmaf(gq.x, v.x, b.x); b.y = fmaf(gq.y, v.y, b.y);
-        b.z = fmaf(gq.z, v.z, b.z); b.w = fmaf(gq.w, v.w, b.w);
-      } else {
-        a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
-        if (kKind == 0) {
-          b.x = fmaf(v.x, v.x, b.x); b.y = fmaf(v.y, v.y, b.y);
-          b.z = fmaf(v.z, v.z, b.z); b.w = fmaf(v.w, v.w, b.w);
+    for (int i0 = threadIdx.x; i0 < hw4; i0 += kThreads * kU) {
+      float4 v[kU], gq[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int i = i0 + kThreads * u;
+        v[u] = i < hw4 ? px[i] : fill;
+        if (kBwd) gq[u] = i < hw4 ? pg[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        float4 d = v[u];
+        d.x -= ref; d.y -= ref; d.z -= ref; d.w -= ref;
+        if (kBwd) {
+          a.x += gq[u].x; a.y += gq[u].y; a.z += gq[u].z; a.w += gq[u].w;
+          b.x = fmaf(gq[u].x, d.x, b.x); b.y = fmaf(gq[u].y, d.y, b.y);
+          b.z = fmaf(gq[u].z, d.z, b.z); b.w = fmaf(gq[u].w, d.w, b.w);
+        } else {
+          a.x += d.x; a.y += d.y; a.z += d.z; a.w += d.w;
+          if (kKind == 0) {
+            b.x = fmaf(d.x, d.x, b.x); b.y = fmaf(d.y, d.y, b.y);
+            b.z = fmaf(d.z, d.z, b.z); b.w = fmaf(d.w, d.w, b.w);
+          }
         }
       }
     }
@@ -218,21 +230,28 @@ template <bool kBwd>
 __device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const float* __restrict__ dy,
                                               float* __restrict__ out, const Geometry& g, int c, int split,
                                               const Coef k) {
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const int hw4 = g.HW >> 2;
   const int n0 = split * g.per_block;
   const int n1 = min(g.N, n0 + g.per_block);
-  for (int n = n1 - 1 - wave; n >= n0; n -= kWaves) {
+  constexpr int kU = kBwd ? 2 : 4;
+  for (int n = n1 - 1; n >= n0; --n) {
     const size_t off = ((size_t)n * g.C + c) * g.HW;
     const float4* __restrict__ px = reinterpret_cast<const float4*>(x + off);
     const float4* __restrict__ pg = reinterpret_cast<const float4*>(dy + (kBwd ? off : 0));
     float4* __restrict__ po = reinterpret_cast<float4*>(out + off);
-#pragma unroll 4
-    for (int i = lane; i < hw4; i += tt::kWave) {
-      const float4 v = px[i];
-      float4 gq = v;
-      if (kBwd) gq = pg[i];
-      po[i] = apply4<kBwd>(v, gq, k);
+    for (int i0 = threadIdx.x; i0 < hw4; i0 += kThreads * kU) {
+      float4 v[kU], gq[kU];
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int i = min(i0 + kThreads * u, hw4 - 1);   // clamped: out-of-range threads re-read, never store
+        v[u] = px[i];
+        gq[u] = kBwd ? pg[i] : v[u];
+      }
+#pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int i = i0 + kThreads * u;
+        if (i < hw4) po[i] = apply4<kBwd>(v[u], gq[u], k);
+      }
     }
   }
 }
@@ -384,14 +403,13 @@ int plan(int N, int C, int HW, Geometry* g, int* mode) {
   g->N = N;
   g->C = C;
   g->HW = HW;
-  const int target_blocks = 4096;  // ~2 resident rounds of 8 blocks on each of 256 CUs
+  const int target_blocks = 16384;  // many short-lived blocks: their start-up and reduction tails overlap other blocks' streaming
   int want = target_blocks / C;
   if (want < 1) want = 1;
   if (want > kMaxSplits) want = kMaxSplits;
   if (HW % 4 == 0 && HW / 4 >= 32) {
     *mode = 0;
     int ppb = ceil_div(N, want);
-    ppb = (ppb + kWaves - 1) / kWaves * kWaves;  // whole rounds of one plane per wave
     g->per_block = ppb;
     g->splits = ceil_div(N, ppb);
     g->hwv_div = tt::make_fastdiv(1);
