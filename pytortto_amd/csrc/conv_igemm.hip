@@ -54,6 +54,13 @@ struct Igemm {
   int ou, ouh, ov, ovw;      // output row = u*ou + ouh, column = v*ov + ovw
   int tilesI;                // row tiles per group
   int tiles;                 // tilesI * pixel tiles
+  // dense input-gradient launches only (all stride-parity classes as rows of one GEMM):
+  // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
+  const int4* rowtab;
+  int outH, outW;
+  // stream-K launches only: the tiles*chunks reduction steps are dealt evenly to the blocks
+  long long skIters;         // tiles * (KQ / kBKQ)
+  floatx4* skPartial;        // [2 * blocks][acc float4s per thread][256] partial accumulators
 };
 
 // ---- preparation kernels (tiny) --------------------------------------------------------------
@@ -121,6 +128,41 @@ __global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ 
   wp[((size_t)g * a.KQ + kq) * a.Ipad + c] = floatx4{v[0], v[1], v[2], v[3]};
 }
 
+// Dense input gradient: every stride-parity class becomes Cg rows of one GEMM over the union
+// of the classes' tap windows.  Row i = (class, c), k = (ko*Na + ia)*Nb + ib reads dy at row
+// offset a = amin + ia from the cell's base row; the weight is w[ko][c][r][s] with
+// r = (ch + ph - a*sh)/dh when that is an integer inside the kernel, else 0 (the class does
+// not have that tap).  Worth it only when Cg is tiny: the zero taps are wasted MACs.
+struct PackDense {
+  int Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, HxWx, Wx;
+};
+__global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restrict__ wp, PackDense a,
+                                   KEntry* __restrict__ tab, KTabArgs ta, int4* __restrict__ rowtab) {
+  const int kq = blockIdx.y;
+  if (blockIdx.x == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= a.Ipad) return;
+  const int cls = i / a.Cg, c = i % a.Cg;
+  const int ch = cls / a.sw, cw = cls % a.sw;
+  if (kq == 0 && i < a.I) rowtab[i] = make_int4(c * a.HxWx + ch * a.Wx + cw, ch, cw, c);
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (i < a.I) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = 4 * kq + j;
+      if (k >= a.Kred) continue;
+      const int ib = k % a.Nb, t = k / a.Nb;
+      const int ia = t % a.Na, ko = t / a.Na;
+      const int rn = ch + a.ph - (a.amin + ia) * a.sh, sn = cw + a.pw - (a.bmin + ib) * a.sw;
+      if (rn < 0 || sn < 0 || rn % a.dh != 0 || sn % a.dw != 0) continue;
+      const int r = rn / a.dh, ss = sn / a.dw;
+      if (r >= a.R || ss >= a.S) continue;
+      v[j] = w[(((size_t)ko * a.Cg + c) * a.R + r) * a.S + ss];
+    }
+  }
+  wp[(size_t)kq * a.Ipad + i] = floatx4{v[0], v[1], v[2], v[3]};
+}
+
 // ---- the GEMM kernel -----------------------------------------------------------------------------
 
 // Blocks are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles, row
@@ -131,12 +173,12 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
 }
 
-template <int WM, int WN, int MT, int NT>
+template <int WM, int WN, int MT, int NT, bool SK>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
-  constexpr int A_ITEMS = kBKQ * BM / kThreads, B_ITEMS = kBKQ * BN / kThreads;
-  static_assert(A_ITEMS >= 1 && B_ITEMS >= 1 && kThreads % BM == 0 && kThreads % BN == 0, "tile shape");
+  constexpr int A_ITEMS = (kBKQ * BM + kThreads - 1) / kThreads, B_ITEMS = kBKQ * BN / kThreads;
+  static_assert(B_ITEMS >= 1 && kThreads % BM == 0 && kThreads % BN == 0, "tile shape");
   __shared__ floatx4 As[2][kBKQ][BM];
   __shared__ floatx4 Bs[2][kBKQ][BN];
 
@@ -144,15 +186,21 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   const int g = blockIdx.y;
-  const int tile = xcd_remap(blockIdx.x, p.tiles);
-  const int i0 = (tile % p.tilesI) * BM;
-  const int m0 = (tile / p.tilesI) * BN;
 
-  // gathered operand: this thread always loads the same pixel, for B_ITEMS k-quads per chunk
+  // gathered operand: within a tile this thread always loads the same pixel, for B_ITEMS
+  // k-quads per chunk
   const int pix = tid % BN;
   const int bq0 = __builtin_amdgcn_readfirstlane(tid / BN);   // first k-quad (wave-uniform)
-  int ih0 = kInvalid, iw0 = 0, base = 0;
-  {
+  const int arow = tid % BM, aq0 = tid / BM;
+  const ConstKTab ktab = (ConstKTab)(uintptr_t)p.ktab;
+  int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0;
+  const floatx4* __restrict__ wsrc = p.wp;
+  auto set_tile = [&](int tile) __attribute__((always_inline)) {
+    i0 = (tile % p.tilesI) * BM;
+    m0 = (tile / p.tilesI) * BN;
+    ih0 = kInvalid;
+    iw0 = 0;
+    base = 0;
     const int m = m0 + pix;
     if (m < p.M) {
       const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
@@ -163,10 +211,8 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       iw0 = (int)v * p.sv + p.bw;
       base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
     }
-  }
-  const ConstKTab ktab = (ConstKTab)(uintptr_t)p.ktab;
-  const floatx4* __restrict__ wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
-  const int arow = tid % BM, aq0 = tid / BM;
+    wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
+  };
 
   floatx4 areg[A_ITEMS];
   floatx4 breg[B_ITEMS];
@@ -174,7 +220,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   constexpr int nB = 4 * B_ITEMS;
   intx2 tab_e[nB];        // table entries {off, dhw} of the chunk being fetched (SGPRs)
 
-  auto load_tab = [&](int chunk) {
+  auto load_tab = [&](int chunk) __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < B_ITEMS; ++it) {
       const int kq = chunk * kBKQ + bq0 + it * (kThreads / BN);
@@ -182,11 +228,11 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       for (int j = 0; j < 4; ++j) tab_e[it * 4 + j] = ktab[kq * 4 + j];
     }
   };
-  auto load_a_item = [&](int chunk, int it) {
-    const int kq = chunk * kBKQ + aq0 + it * (kThreads / BM);
-    areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
+  auto load_a_item = [&](int chunk, int it) __attribute__((always_inline)) {
+    const int q = aq0 + it * (kThreads / BM);   // always < kBKQ unless the tile has fewer than 64 rows
+    if (q < kBKQ) areg[it] = wsrc[(size_t)(chunk * kBKQ + q) * p.Ipad + arow];
   };
-  auto load_b_elem = [&](int e) {   // uses tab_e: must follow load_tab() of the same chunk
+  auto load_b_elem = [&](int e) __attribute__((always_inline)) {   // uses tab_e: must follow load_tab() of the same chunk
     const intx2 t = tab_e[e];
     const int ih = ih0 + (int)(short)(t.y & 0xffff);
     const int iw = iw0 + (t.y >> 16);
@@ -195,8 +241,11 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     breg[e >> 2][e & 3] = p.src[off];
     bok[e >> 2][e & 3] = ok;
   };
-  auto store_a_item = [&](int buf, int it) { As[buf][aq0 + it * (kThreads / BM)][arow] = areg[it]; };
-  auto store_b_item = [&](int buf, int it) {
+  auto store_a_item = [&](int buf, int it) __attribute__((always_inline)) {
+    const int q = aq0 + it * (kThreads / BM);
+    if (q < kBKQ) As[buf][q][arow] = areg[it];
+  };
+  auto store_b_item = [&](int buf, int it) __attribute__((always_inline)) {
     floatx4 v;
 #pragma unroll
     for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
@@ -206,7 +255,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   // MFMA operands of one chunk: [kk][tile] float4 = four k-steps each.  Lanes 0-31 take quad
   // 2*kk, lanes 32-63 quad 2*kk+1, so MFMA step j of half kk contracts k = 4*(2*kk + h) + j.
   floatx4 opA[2][2][MT], opB[2][2][NT];
-  auto read_ops = [&](int set, int buf) {
+  auto read_ops = [&](int set, int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
@@ -217,12 +266,6 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   };
 
   floatx16 acc[MT][NT];
-#pragma unroll
-  for (int a = 0; a < MT; ++a)
-#pragma unroll
-    for (int b = 0; b < NT; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   // One chunk of MFMAs (operand set `set`, read from LDS buffer `set` earlier) with the work for
   // the following chunks woven in between them, one small step per MFMA, so that it executes in
@@ -233,7 +276,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   //                    scalar loads of the table entries of chunk `nnchunk`
   // sched_barrier pins this order; the compiler otherwise sinks the loads below the MFMAs.
   constexpr int T = 8 * MT * NT;
-  auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) {
+  auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
     if constexpr (T >= 32) {
       constexpr int kStore = T - 8, kSync = T - 4;
       static_assert(nB + A_ITEMS <= kStore && kStore + B_ITEMS + A_ITEMS - 1 <= kSync, "schedule does not fit");
@@ -277,58 +320,183 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     }
   };
 
-  const int chunks = p.KQ / kBKQ;
-  if (chunks > 0) {
-    load_tab(0);
+  // Reduction chunks [c0, c1) of the current tile into acc (zeroed first).
+  auto run_segment = [&](const int c0, const int c1) __attribute__((always_inline)) {
+#pragma unroll
+    for (int a = 0; a < MT; ++a)
+#pragma unroll
+      for (int b = 0; b < NT; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+    if (c0 >= c1) return;
+    const int last = c1 - 1;
+    load_tab(c0);
 #pragma unroll
     for (int e = 0; e < nB; ++e) load_b_elem(e);
 #pragma unroll
-    for (int it = 0; it < A_ITEMS; ++it) load_a_item(0, it);
+    for (int it = 0; it < A_ITEMS; ++it) load_a_item(c0, it);
 #pragma unroll
     for (int it = 0; it < B_ITEMS; ++it) store_b_item(0, it);
 #pragma unroll
     for (int it = 0; it < A_ITEMS; ++it) store_a_item(0, it);
     __syncthreads();
     read_ops(0, 0);
-    load_tab(min(1, chunks - 1));
-    // the last chunks re-fetch the final chunk (cache hits) instead of branching: a loop body
+    load_tab(min(c0 + 1, last));
+    // the final chunks re-fetch the last chunk (cache hits) instead of branching: a loop body
     // free of conditions keeps the prefetch registers in registers
-    int c = 0;
-    for (; c + 1 < chunks; c += 2) {
-      chunk_body(0, c + 1, min(c + 2, chunks - 1));
-      chunk_body(1, min(c + 2, chunks - 1), min(c + 3, chunks - 1));
+    int c = c0;
+    for (; c + 1 < c1; c += 2) {
+      chunk_body(0, c + 1, min(c + 2, last));
+      chunk_body(1, min(c + 2, last), min(c + 3, last));
     }
-    if (c < chunks) chunk_body(0, c, c);
-  }
+    if (c < c1) chunk_body(0, c, c);
+  };
 
   // epilogue: accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*h + r%4, column l32
-  uint32_t obase[NT];
-  bool mok[NT];
+  auto epilogue = [&]() __attribute__((always_inline)) {
+    uint32_t obase[NT];
+    bool mok[NT];
+#pragma unroll
+    for (int y = 0; y < NT; ++y) {
+      const int m = m0 + (wn * NT + y) * 32 + l32;
+      mok[y] = m < p.M;
+      const uint32_t mm = mok[y] ? (uint32_t)m : 0u;
+      const uint32_t n = tt::fd_div(mm, p.divUV);
+      const uint32_t rem = mm - n * p.divUV.d;
+      const uint32_t u = tt::fd_div(rem, p.divV);
+      const uint32_t v = rem - u * p.divV.d;
+      obase[y] = (uint32_t)((int)n * p.outStrideN + g * p.outStrideG + ((int)u * p.ou + p.ouh) * p.outRow +
+                            (int)v * p.ov + p.ovw);
+    }
+    if (p.rowtab == nullptr) {
+#pragma unroll
+      for (int x = 0; x < MT; ++x) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+          if (i < p.I) {
+            const float bz = p.bias ? p.bias[g * p.I + i] : 0.f;
+            const uint32_t ioff = (uint32_t)(i * p.outStrideI);
+#pragma unroll
+            for (int y = 0; y < NT; ++y)
+              if (mok[y]) p.out[obase[y] + ioff] = acc[x][y][r] + bz;
+          }
+        }
+      }
+    } else {
+      // rows are (parity class, channel): each row has its own offset inside the sh x sw cell
+      // anchored at the pixel, and cells at the bottom/right edge may be cut off
+      int oh[NT], ow[NT];
+#pragma unroll
+      for (int y = 0; y < NT; ++y) {
+        const int m = m0 + (wn * NT + y) * 32 + l32;
+        const uint32_t mm = mok[y] ? (uint32_t)m : 0u;
+        const uint32_t rem = mm - tt::fd_div(mm, p.divUV) * p.divUV.d;
+        const uint32_t u = tt::fd_div(rem, p.divV);
+        oh[y] = (int)u * p.ou;
+        ow[y] = (int)(rem - u * p.divV.d) * p.ov;
+      }
+#pragma unroll
+      for (int x = 0; x < MT; ++x) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+          if (i < p.I) {
+            const int4 e = p.rowtab[i];
+            const float bz = p.bias ? p.bias[e.w] : 0.f;
+#pragma unroll
+            for (int y = 0; y < NT; ++y)
+              if (mok[y] && oh[y] + e.y < p.outH && ow[y] + e.z < p.outW)
+                p.out[obase[y] + (uint32_t)e.x] = acc[x][y][r] + bz;
+          }
+        }
+      }
+    }
+  };
+
+  const int chunks = p.KQ / kBKQ;
+  if constexpr (!SK) {
+    set_tile(xcd_remap(blockIdx.x, p.tiles));
+    run_segment(0, chunks);
+    epilogue();
+  } else {
+    // Stream-K: block b owns reduction steps [b*T/P, (b+1)*T/P) of the tile-major sequence of
+    // all T = tiles*chunks steps, so every block does the same amount of MFMA work whatever
+    // the number of tiles.  A tile covered by one block is finished here; otherwise each block
+    // leaves its partial accumulators (slot 2b if it entered the tile mid-way, 2b+1 if it
+    // started the tile but does not finish it) and igemm_fixup adds them in block order.
+    constexpr int kAccQ = MT * NT * 4;
+    const int nblk = gridDim.x;
+    const int b = xcd_remap(blockIdx.x, nblk);
+    long long it = (long long)b * p.skIters / nblk;
+    const long long end = (long long)(b + 1) * p.skIters / nblk;
+    while (it < end) {
+      const int tile = (int)(it / chunks);
+      const int c0 = (int)(it - (long long)tile * chunks);
+      const int n = (int)min((long long)(chunks - c0), end - it);
+      set_tile(tile);
+      run_segment(c0, c0 + n);
+      if (n == chunks) {
+        epilogue();
+      } else {
+        floatx4* __restrict__ dst = p.skPartial + ((size_t)(2 * b + (c0 == 0 ? 1 : 0)) * kAccQ) * kThreads + tid;
+#pragma unroll
+        for (int x = 0; x < MT; ++x)
+#pragma unroll
+          for (int y = 0; y < NT; ++y)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              dst[(size_t)((x * NT + y) * 4 + q) * kThreads] =
+                  floatx4{acc[x][y][4 * q], acc[x][y][4 * q + 1], acc[x][y][4 * q + 2], acc[x][y][4 * q + 3]};
+      }
+      it += n;
+      __syncthreads();   // the next segment's first stores reuse LDS buffer 0
+    }
+  }
+}
+
+// Stream-K second stage: one block per tile; tiles that a single block computed are already
+// stored, the others are the sum of their segments' partial accumulators (added in block
+// order, so the result does not depend on timing), plus bias.
+template <int WM, int WN, int MT, int NT>
+__global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p, int nblk) {
+  constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
+  constexpr int kAccQ = MT * NT * 4;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = tid >> 6, wm = wave / WN, wn = wave % WN;
+  const int tile = blockIdx.x;
+  const int chunks = p.KQ / kBKQ;
+  const long long t0 = (long long)tile * chunks, t1 = t0 + chunks;
+  // block containing step s: the largest b with b*T/P <= s
+  const int b_first = (int)(((t0 + 1) * nblk - 1) / p.skIters);
+  const int b_last = (int)((t1 * nblk - 1) / p.skIters);
+  if (b_first == b_last) return;
+  floatx4 acc[kAccQ];
+#pragma unroll
+  for (int q = 0; q < kAccQ; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int b = b_first; b <= b_last; ++b) {
+    const long long begin = (long long)b * p.skIters / nblk;
+    const floatx4* __restrict__ src = p.skPartial + ((size_t)(2 * b + (begin > t0 ? 0 : 1)) * kAccQ) * kThreads + tid;
+#pragma unroll
+    for (int q = 0; q < kAccQ; ++q) acc[q] += src[(size_t)q * kThreads];
+  }
+  const int i0 = (tile % p.tilesI) * BM, m0 = (tile / p.tilesI) * BN;
 #pragma unroll
   for (int y = 0; y < NT; ++y) {
     const int m = m0 + (wn * NT + y) * 32 + l32;
-    mok[y] = m < p.M;
-    const uint32_t mm = mok[y] ? (uint32_t)m : 0u;
-    const uint32_t n = tt::fd_div(mm, p.divUV);
-    const uint32_t rem = mm - n * p.divUV.d;
+    if (m >= p.M) continue;
+    const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
+    const uint32_t rem = (uint32_t)m - n * p.divUV.d;
     const uint32_t u = tt::fd_div(rem, p.divV);
     const uint32_t v = rem - u * p.divV.d;
-    obase[y] = (uint32_t)((int)n * p.outStrideN + g * p.outStrideG + ((int)u * p.ou + p.ouh) * p.outRow +
-                          (int)v * p.ov + p.ovw);
-  }
+    const uint32_t obase = (uint32_t)((int)n * p.outStrideN + ((int)u * p.ou + p.ouh) * p.outRow + (int)v * p.ov + p.ovw);
 #pragma unroll
-  for (int x = 0; x < MT; ++x) {
+    for (int x = 0; x < MT; ++x)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (i < p.I) {
-        const float bz = p.bias ? p.bias[g * p.I + i] : 0.f;
-        const uint32_t ioff = (uint32_t)(i * p.outStrideI);
-#pragma unroll
-        for (int y = 0; y < NT; ++y)
-          if (mok[y]) p.out[obase[y] + ioff] = acc[x][y][r] + bz;
+      for (int r = 0; r < 16; ++r) {
+        const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[(x * NT + y) * 4 + (r >> 2)][r & 3] + (p.bias ? p.bias[i] : 0.f);
       }
-    }
   }
 }
 
@@ -339,39 +507,69 @@ int gcd(int a, int b) { return b == 0 ? a : gcd(b, a % b); }
 
 struct TileChoice {
   int bm, bn;
+  int sk_blocks;   // > 0: stream-K launch with this many blocks
 };
 
-// 128x128 by default; 64 rows when a group has no more than 64 of them; 64x64 when the bigger
-// tiles would leave most of the 256 CUs idle.
-TileChoice choose_tile(int I, int M, int groups) {
+constexpr int kCUs = 256;             // MI355X
+constexpr int kSkBlocks = 2 * kCUs;   // two co-resident blocks per CU
+
+// Stream-K pays (a second small kernel, partial tiles through HBM) and only helps when the
+// tiles do not spread evenly over the CUs; it needs a reduction long enough to split.
+bool wants_stream_k(long long tiles, int chunks, int groups) {
+  if (groups != 1 || chunks < 8) return false;
+  if (tiles * chunks < 4LL * kSkBlocks) return false;
+  const long long rounds = (tiles + kCUs - 1) / kCUs;
+  return (double)tiles / (double)(rounds * kCUs) < 0.93;
+}
+
+// 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
+// CUs idle or unevenly loaded the reduction is split stream-K fashion; if it is too short for
+// that, 64x64 tiles raise the block count instead.
+TileChoice choose_tile(int I, int M, int groups, int chunks) {
   TileChoice t;
-  if (I <= 64) {
-    t.bm = 64;
-    t.bn = 256;
-  } else {
-    t.bm = 128;
-    t.bn = 128;
-  }
-  const long long blocks = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn) * groups;
-  if (blocks < 256) {
+  t.bm = I <= 64 ? 64 : 128;
+  t.bn = I <= 64 ? 256 : 128;
+  t.sk_blocks = 0;
+  const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
+  if (wants_stream_k(tiles, chunks, groups)) {
+    t.sk_blocks = kSkBlocks;
+  } else if (tiles * groups < kCUs) {
     t.bm = 64;
     t.bn = 64;
+    const long long small = (long long)ceil_div(I, 64) * ceil_div(M, 64);
+    if (wants_stream_k(small, chunks, groups)) t.sk_blocks = kSkBlocks;
   }
   return t;
 }
 
-int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id) {
+// bytes of stream-K partial accumulators for the largest tile: 2 slots per block
+size_t sk_workspace_bytes() { return (size_t)2 * kSkBlocks * 128 * 128 * sizeof(float); }
+
+template <int WM, int WN, int MT, int NT>
+void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+  if (sk_blocks > 0) {
+    igemm_f32<WM, WN, MT, NT, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    igemm_fixup<WM, WN, MT, NT><<<p.tiles, kThreads, 0, st>>>(p, sk_blocks);
+  } else {
+    igemm_f32<WM, WN, MT, NT, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+  }
+}
+
+int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_partial) {
   tt::ProfScope prof(prof_id);
   p.tilesI = p.Ipad / t.bm;
   p.tiles = p.tilesI * ceil_div(p.M, t.bn);
-  dim3 grid(p.tiles, groups);
+  p.skIters = (long long)p.tiles * (p.KQ / kBKQ);
+  p.skPartial = sk_partial;
   hipStream_t st = tt::stream();
   if (t.bm == 128 && t.bn == 128)
-    igemm_f32<2, 2, 2, 2><<<grid, kThreads, 0, st>>>(p);
+    launch_config<2, 2, 2, 2>(p, groups, t.sk_blocks, st);
   else if (t.bm == 64 && t.bn == 256)
-    igemm_f32<1, 4, 2, 2><<<grid, kThreads, 0, st>>>(p);
+    launch_config<1, 4, 2, 2>(p, groups, t.sk_blocks, st);
+  else if (t.bm == 32 && t.bn == 256)
+    launch_config<1, 4, 1, 2>(p, groups, t.sk_blocks, st);
   else
-    igemm_f32<2, 2, 1, 1><<<grid, kThreads, 0, st>>>(p);
+    launch_config<2, 2, 1, 1>(p, groups, t.sk_blocks, st);
   TT_LAUNCH_CHECK();
   return 0;
 }
@@ -411,14 +609,14 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   const int Cg = C / groups, Kg = K / groups;
   const int Kred = Cg * R * S;
   const int M = N * P * Q;
-  const TileChoice t = choose_tile(Kg, M, groups);
-  const int Ipad = ceil_div(Kg, t.bm) * t.bm;
   const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
+  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ);
+  const int Ipad = ceil_div(Kg, t.bm) * t.bm;
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
-  const size_t tab_bytes = sizeof(KEntry) * (size_t)KQ * 4;
+  const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
   void* ws;
-  if (tt::workspace(wp_bytes + tab_bytes, &ws)) return -1;
+  if (tt::workspace(wp_bytes + tab_bytes + sk_workspace_bytes(), &ws)) return -1;
   floatx4* wp = (floatx4*)ws;
   KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
   hipStream_t st = tt::stream();
@@ -439,7 +637,7 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   p.srcStrideN = C * H * W; p.srcStrideG = Cg * H * W;
   p.outStrideN = K * P * Q; p.outStrideG = Kg * P * Q; p.outStrideI = P * Q; p.outRow = Q;
   p.ou = 1; p.ouh = 0; p.ov = 1; p.ovw = 0;
-  return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD);
+  return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes + tab_bytes));
 }
 
 int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
@@ -453,17 +651,78 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
   const int rstep = sh / gh, sstep = sw / gw;   // valid taps of a class: r0, r0+rstep, ...
   const int eh = dh / gh, ew = dw / gw;          // dy row/column step per tap
 
+  const int classes = sh * sw;
+  TT_REQUIRE(classes <= 4096, "tt_conv2d_dgrad_f32: stride %d x %d not supported", sh, sw);
+  hipStream_t st = tt::stream();
+
+  if (groups == 1 && classes > 1 && classes * Cg <= 64 && Hx >= sh && Wx >= sw) {
+    // tiny Cg: per-class GEMMs would fill 3 of 32 MFMA rows; stack all classes as rows instead
+    int amin = 1 << 30, amax = -(1 << 30), bmin = 1 << 30, bmax = -(1 << 30);
+    for (int ch = 0; ch < sh; ++ch)
+      for (int r = 0; r < R; ++r)
+        if (((ch + ph - r * dh) % sh + sh) % sh == 0) {
+          const int a = (ch + ph - r * dh) / sh;   // exact
+          amin = a < amin ? a : amin;
+          amax = a > amax ? a : amax;
+        }
+    for (int cw = 0; cw < sw; ++cw)
+      for (int s2 = 0; s2 < S; ++s2)
+        if (((cw + pw - s2 * dw) % sw + sw) % sw == 0) {
+          const int b = (cw + pw - s2 * dw) / sw;
+          bmin = b < bmin ? b : bmin;
+          bmax = b > bmax ? b : bmax;
+        }
+    if (amin <= amax && bmin <= bmax) {
+      const int Na = amax - amin + 1, Nb = bmax - bmin + 1;
+      const int I = classes * Cg;
+      const int Kred = Kg * Na * Nb;
+      const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
+      const int U = ceil_div(Hx, sh), V = ceil_div(Wx, sw);
+      const int M = N * U * V;
+      TileChoice t;
+      t.bm = I <= 32 ? 32 : 64;
+      t.bn = 256;
+      t.sk_blocks = 0;
+      const int Ipad = t.bm;
+      const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)KQ * Ipad, 256);
+      const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
+      const size_t row_bytes = align_up(sizeof(int4) * (size_t)I, 256);
+      void* ws;
+      if (tt::workspace(wp_bytes + tab_bytes + row_bytes, &ws)) return -1;
+      floatx4* wp = (floatx4*)ws;
+      KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
+      int4* rowtab = (int4*)((char*)ws + wp_bytes + tab_bytes);
+      {
+        tt::ProfScope prof(TT_PROF_CONV_PREP);
+        PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx};
+        KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1};
+        pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa, tab, ka, rowtab);
+        TT_LAUNCH_CHECK();
+      }
+      Igemm p{};
+      p.src = dy; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.I = I; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
+      p.divUV = tt::make_fastdiv((uint32_t)(U * V));
+      p.divV = tt::make_fastdiv((uint32_t)V);
+      p.su = 1; p.bh = amin; p.sv = 1; p.bw = bmin;
+      p.Hlim = P; p.Wlim = Q; p.srcRow = Q;
+      p.srcStrideN = K * P * Q; p.srcStrideG = 0;
+      p.outStrideN = C * Hx * Wx; p.outStrideG = 0; p.outStrideI = 0; p.outRow = Wx;
+      p.ou = sh; p.ouh = 0; p.ov = sw; p.ovw = 0;
+      p.rowtab = rowtab; p.outH = Hx; p.outW = Wx;
+      return launch_igemm(p, 1, t, TT_PROF_CONV_IGEMM_DGRAD, nullptr);
+    }
+  }
+
   // workspace: the largest class (all taps at stride 1) bounds every class
   int max_taps_r = ceil_div(R, rstep), max_taps_s = ceil_div(S, sstep);
   const int KQmax = ceil_div((long long)Kg * max_taps_r * max_taps_s, 4 * kBKQ) * kBKQ;
   const int IpadMax = ceil_div(Cg, 128) * 128;
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQmax * IpadMax, 256);
   const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQmax * 4, 256);
-  const int classes = sh * sw;
-  TT_REQUIRE(classes <= 4096, "tt_conv2d_dgrad_f32: stride %d x %d not supported", sh, sw);
   void* ws;
-  if (tt::workspace((wp_bytes + tab_bytes) * classes, &ws)) return -1;
-  hipStream_t st = tt::stream();
+  if (tt::workspace((wp_bytes + tab_bytes) * classes + sk_workspace_bytes(), &ws)) return -1;
+  floatx4* sk_partial = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * classes);
 
   int slot = 0;
   for (int ch = 0; ch < sh && ch < Hx; ++ch) {
@@ -481,9 +740,9 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       const int V = ceil_div(Wx - cw, sw);
       const int Kred = Kg * nTr * nTs;
       const int M = N * U * V;
-      const TileChoice t = choose_tile(Cg, M, groups);
-      const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
+      const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ);
+      const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
       Igemm p{};
@@ -506,7 +765,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       p.srcStrideN = K * P * Q; p.srcStrideG = Kg * P * Q;
       p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
       p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
-      if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD)) return -1;
+      if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
     }
   }
   return 0;

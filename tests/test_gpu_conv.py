@@ -69,6 +69,9 @@ TILE_CASES = [
     (2, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # small M, long reduction
     (4, 64, 20, 20, 96, 3, 3, (1, 1), (2, 2), (2, 2), 4),       # groups + dilation
     (128, 4, 64, 64, 16, 3, 2, (1, 3), (2, 3), (1, 2), 2),      # the reference notebook's configuration
+    (8, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # 49 tiles of 128x128: split reduction (stream-K)
+    (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # 196 tiles of 64x256: stream-K
+    (8, 256, 14, 14, 256, 3, 3, (2, 2), (1, 1), (1, 1), 1),     # stream-K in every dgrad parity class
 ]
 
 
