@@ -241,6 +241,10 @@ def main():
     del bns
     call('tt_empty_cache')
 
+    # ---- what the device sustains on the two bounding resources, measured in this run ----------
+    mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
+    hbm_read, hbm_copy = _hip.probe_hbm(2 << 30)
+
     # ---- CPU baseline (oracle on the host cores) -------------------------------------------------
     cpu_conv = cpu_bn = None
     if not args.no_cpu_baseline:
@@ -268,6 +272,10 @@ def main():
         'roofline': {'bound': 'mfma', 'kernel': 'igemm_f32 (Conv2d forward + input gradient)',
                      'achieved': round(igemm_tflops, 2), 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(igemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4), 'traffic': None,
+                     'sustained_peak_measured': {'mean': round(mfma_mean, 1), 'min': round(mfma_min, 1),
+                                                 'max': round(mfma_max, 1), 'unit': 'TFLOP/s',
+                                                 'what': '100 launches of dense v_mfma_f32_32x32x2_f32, '
+                                                         'per-lane varying operands'},
                      'launches_per_step': (n_fwd + n_dg) // args.steps,
                      'avg_launch_ms': round((ms_fwd + ms_dg) / max(1, n_fwd + n_dg), 5)},
         'kernels_ms_per_step': kernel_ms,
@@ -282,6 +290,8 @@ def main():
                'roofline': {'bound': 'hbm', 'kernel': 'bn_bwd_apply (reads x, dy; writes dx)',
                             'achieved': round(bwd_apply_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                             'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4), 'traffic': None,
+                            'sustained_measured': {'read_gbs': round(hbm_read, 1), 'copy_gbs': round(hbm_copy, 1),
+                                                   'what': '2 GiB streamed, 16 KiB contiguous per block'},
                             'avg_launch_ms': round(ms_ba / max(1, n_ba), 5)},
                'kernels_ms_per_step': bn_kernel_ms,
                'cpu_baseline': cpu_bn},

@@ -70,6 +70,14 @@ enum {
 int tt_profile_enable(int on);
 int tt_profile_read(int kernel_id, long long* launches, double* total_ms);
 
+/* Calibration probes (no counterpart in the reference): what the device sustains with nothing
+ * else in the way.  tt_probe_mfma_f32 runs `launches` back-to-back launches (about 1.3 ms each)
+ * of dense v_mfma_f32_32x32x2_f32 with per-lane varying operands and reports TFLOP/s (host
+ * pointers); tt_probe_hbm_f32 streams `bytes` (>= 64 MiB) with 16 KiB contiguous chunks per
+ * block: read-only GB/s and copy GB/s (read + written bytes). */
+int tt_probe_mfma_f32(int launches, double* tflops_mean, double* tflops_min, double* tflops_max);
+int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
+
 /* ---- convolution ------------------------------------------------------------------------- */
 
 /* y[N,K,P,Q] = conv(x[N,C,H,W], w[K,C/groups,R,S]) (+ bias[K] if not NULL).

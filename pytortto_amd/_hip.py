@@ -32,6 +32,8 @@ PROTOTYPES = {
     'tt_event_destroy': [_P],
     'tt_profile_enable': [_I],
     'tt_profile_read': [_I, POINTER(ctypes.c_longlong), POINTER(c_double)],
+    'tt_probe_mfma_f32': [_I, POINTER(c_double), POINTER(c_double), POINTER(c_double)],
+    'tt_probe_hbm_f32': [c_size_t, POINTER(c_double), POINTER(c_double)],
     'tt_conv2d_fwd_f32': [_P, _P, _P, _P] + [_I] * 14,
     'tt_conv2d_dgrad_f32': [_P, _P, _P, _P] + [_I] * 16,
     'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
@@ -124,6 +126,20 @@ def profile_read():
         call('tt_profile_read', kid, ctypes.byref(n), ctypes.byref(ms))
         out[name] = (n.value, ms.value)
     return out
+
+
+def probe_mfma(launches=100):
+    """Sustained dense fp32 MFMA TFLOP/s: (mean, min, max) over ``launches`` launches."""
+    mean, lo, hi = c_double(), c_double(), c_double()
+    call('tt_probe_mfma_f32', launches, ctypes.byref(mean), ctypes.byref(lo), ctypes.byref(hi))
+    return mean.value, lo.value, hi.value
+
+
+def probe_hbm(nbytes=2 << 30):
+    """Streaming bandwidth in GB/s: (read only, copy counting read + written bytes)."""
+    rd, cp = c_double(), c_double()
+    call('tt_probe_hbm_f32', nbytes, ctypes.byref(rd), ctypes.byref(cp))
+    return rd.value, cp.value
 
 
 def synchronize():
