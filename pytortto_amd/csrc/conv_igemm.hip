@@ -59,8 +59,10 @@ struct Igemm {
   const int4* rowtab;
   int outH, outW;
   // stream-K launches only: the tiles*chunks reduction steps are dealt evenly to the blocks
-  long long skIters;         // tiles * (KQ / kBKQ)
-  floatx4* skPartial;        // [2 * blocks][acc float4s per thread][256] partial accumulators
+  int skDpTiles;             // tiles [0, skDpTiles) are computed whole, block b takes b, b+blocks, ...
+  int skBlocks;              // blocks that share the remaining tiles' reduction steps
+  long long skIters;         // (tiles - skDpTiles) * (KQ / kBKQ)
+  floatx4* skPartial;        // [2 * skBlocks][acc float4s per thread][256] partial accumulators
 };
 
 // ---- preparation kernels (tiny) --------------------------------------------------------------
@@ -420,37 +422,47 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     run_segment(0, chunks);
     epilogue();
   } else {
-    // Stream-K: block b owns reduction steps [b*T/P, (b+1)*T/P) of the tile-major sequence of
-    // all T = tiles*chunks steps, so every block does the same amount of MFMA work whatever
-    // the number of tiles.  A tile covered by one block is finished here; otherwise each block
-    // leaves its partial accumulators (slot 2b if it entered the tile mid-way, 2b+1 if it
-    // started the tile but does not finish it) and igemm_fixup adds them in block order.
+    // Whole rounds of tiles are computed one tile per block as usual.  The tiles left over would
+    // load the CUs unevenly, so their reduction steps (tile-major sequence of T = tiles*chunks
+    // steps) are dealt evenly instead: block b owns steps [b*T/P, (b+1)*T/P).  A left-over tile
+    // covered by one block is finished here; otherwise each block leaves its partial
+    // accumulators (slot 2b if it entered the tile mid-way, 2b+1 if it started the tile but does
+    // not finish it) and igemm_fixup adds them in block order.  (Letting the last block to
+    // arrive do that sum inside this kernel was tried: the device-scope fences it needs write
+    // back and invalidate whole L2s on this multi-die part and cost more than the second launch.)
     constexpr int kAccQ = MT * NT * 4;
-    const int nblk = gridDim.x;
-    const int b = xcd_remap(blockIdx.x, nblk);
-    long long it = (long long)b * p.skIters / nblk;
-    const long long end = (long long)(b + 1) * p.skIters / nblk;
-    while (it < end) {
-      const int tile = (int)(it / chunks);
-      const int c0 = (int)(it - (long long)tile * chunks);
-      const int n = (int)min((long long)(chunks - c0), end - it);
+    const int b = xcd_remap(blockIdx.x, gridDim.x);
+    for (int tile = b; tile < p.skDpTiles; tile += gridDim.x) {
       set_tile(tile);
-      run_segment(c0, c0 + n);
-      if (n == chunks) {
-        epilogue();
-      } else {
-        floatx4* __restrict__ dst = p.skPartial + ((size_t)(2 * b + (c0 == 0 ? 1 : 0)) * kAccQ) * kThreads + tid;
+      run_segment(0, chunks);
+      epilogue();
+      __syncthreads();   // the next tile's first stores reuse LDS buffer 0
+    }
+    if (b < p.skBlocks) {
+      long long it = (long long)b * p.skIters / p.skBlocks;
+      const long long end = (long long)(b + 1) * p.skIters / p.skBlocks;
+      while (it < end) {
+        const int t = (int)(it / chunks);
+        const int c0 = (int)(it - (long long)t * chunks);
+        const int n = (int)min((long long)(chunks - c0), end - it);
+        set_tile(p.skDpTiles + t);
+        run_segment(c0, c0 + n);
+        if (n == chunks) {
+          epilogue();
+        } else {
+          floatx4* __restrict__ dst = p.skPartial + ((size_t)(2 * b + (c0 == 0 ? 1 : 0)) * kAccQ) * kThreads + tid;
 #pragma unroll
-        for (int x = 0; x < MT; ++x)
+          for (int x = 0; x < MT; ++x)
 #pragma unroll
-          for (int y = 0; y < NT; ++y)
+            for (int y = 0; y < NT; ++y)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              dst[(size_t)((x * NT + y) * 4 + q) * kThreads] =
-                  floatx4{acc[x][y][4 * q], acc[x][y][4 * q + 1], acc[x][y][4 * q + 2], acc[x][y][4 * q + 3]};
+              for (int q = 0; q < 4; ++q)
+                dst[(size_t)((x * NT + y) * 4 + q) * kThreads] =
+                    floatx4{acc[x][y][4 * q], acc[x][y][4 * q + 1], acc[x][y][4 * q + 2], acc[x][y][4 * q + 3]};
+        }
+        it += n;
+        __syncthreads();
       }
-      it += n;
-      __syncthreads();   // the next segment's first stores reuse LDS buffer 0
     }
   }
 }
@@ -459,14 +471,15 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
 // stored, the others are the sum of their segments' partial accumulators (added in block
 // order, so the result does not depend on timing), plus bias.
 template <int WM, int WN, int MT, int NT>
-__global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p, int nblk) {
+__global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p) {
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int kAccQ = MT * NT * 4;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = tid >> 6, wm = wave / WN, wn = wave % WN;
-  const int tile = blockIdx.x;
+  const int tile = p.skDpTiles + blockIdx.x;   // one block per left-over tile
+  const int nblk = p.skBlocks;
   const int chunks = p.KQ / kBKQ;
-  const long long t0 = (long long)tile * chunks, t1 = t0 + chunks;
+  const long long t0 = (long long)blockIdx.x * chunks, t1 = t0 + chunks;
   // block containing step s: the largest b with b*T/P <= s
   const int b_first = (int)(((t0 + 1) * nblk - 1) / p.skIters);
   const int b_last = (int)((t1 * nblk - 1) / p.skIters);
@@ -507,7 +520,7 @@ int gcd(int a, int b) { return b == 0 ? a : gcd(b, a % b); }
 
 struct TileChoice {
   int bm, bn;
-  int sk_blocks;   // > 0: stream-K launch with this many blocks
+  int sk_blocks;   // > 0: persistent launch with this many blocks, left-over tiles split stream-K fashion
 };
 
 constexpr int kCUs = 256;             // MI355X
@@ -549,7 +562,7 @@ template <int WM, int WN, int MT, int NT>
 void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   if (sk_blocks > 0) {
     igemm_f32<WM, WN, MT, NT, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
-    igemm_fixup<WM, WN, MT, NT><<<p.tiles, kThreads, 0, st>>>(p, sk_blocks);
+    igemm_fixup<WM, WN, MT, NT><<<p.tiles - p.skDpTiles, kThreads, 0, st>>>(p);
   } else {
     igemm_f32<WM, WN, MT, NT, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
@@ -559,8 +572,21 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
   tt::ProfScope prof(prof_id);
   p.tilesI = p.Ipad / t.bm;
   p.tiles = p.tilesI * ceil_div(p.M, t.bn);
-  p.skIters = (long long)p.tiles * (p.KQ / kBKQ);
-  p.skPartial = sk_partial;
+  if (t.sk_blocks > 0) {
+    const int chunks = p.KQ / kBKQ;
+    const int rem = p.tiles % t.sk_blocks;
+    if (rem == 0) {
+      t.sk_blocks = 0;   // whole rounds only: nothing to split
+    } else {
+      p.skDpTiles = p.tiles - rem;
+      p.skIters = (long long)rem * chunks;
+      // every sharing block gets at least 8 reduction steps of work for the partial tile it leaves
+      long long share = p.skIters / 8;
+      if (share < rem) share = rem;
+      p.skBlocks = (int)(share < t.sk_blocks ? share : t.sk_blocks);
+      p.skPartial = sk_partial;
+    }
+  }
   hipStream_t st = tt::stream();
   if (t.bm == 128 && t.bn == 128)
     launch_config<2, 2, 2, 2>(p, groups, t.sk_blocks, st);
