@@ -54,6 +54,9 @@ struct Igemm {
   int ou, ouh, ov, ovw;      // output row = u*ou + ouh, column = v*ov + ovw
   int tilesI;                // row tiles per group
   int tiles;                 // tilesI * pixel tiles
+  // plain-GEMM launches only (1x1, stride 1, no padding: the gathered operand is the [k][pixel]
+  // matrix itself): elements between consecutive k rows, and the real reduction length
+  int kStride, Kred;
   // dense input-gradient launches only (all stride-parity classes as rows of one GEMM):
   // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
   const int4* rowtab;
@@ -175,7 +178,7 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
 }
 
-template <int WM, int WN, int MT, int NT, bool SK>
+template <int WM, int WN, int MT, int NT, bool SK, bool GEMM>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
@@ -195,7 +198,9 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   const int bq0 = __builtin_amdgcn_readfirstlane(tid / BN);   // first k-quad (wave-uniform)
   const int arow = tid % BM, aq0 = tid / BM;
   const ConstKTab ktab = (ConstKTab)(uintptr_t)p.ktab;
-  int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0;
+  constexpr int GPQ = BN / 4, GR = BN / 64;
+  const int gpq = tid % GPQ, gkr = (tid / GPQ) * GR;
+  int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0, gbase = 0;
   const floatx4* __restrict__ wsrc = p.wp;
   auto set_tile = [&](int tile) __attribute__((always_inline)) {
     i0 = (tile % p.tilesI) * BM;
@@ -214,6 +219,35 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
     }
     wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
+    if constexpr (GEMM) {
+      // four consecutive pixels per thread: m % 4 == 0 and (U*V) % 4 == 0, so they share n
+      const int mq = min(m0 + 4 * gpq, p.M - 4);   // past-the-end quads re-read the last one; never stored
+      const uint32_t n = tt::fd_div((uint32_t)mq, p.divUV);
+      gbase = (int)n * p.srcStrideN + g * p.srcStrideG + (int)((uint32_t)mq - n * p.divUV.d);
+    }
+  };
+
+  // plain-GEMM mode: thread (gpq, gkr) loads rows gkr .. gkr+GR-1 of the chunk's 16 k rows for
+  // pixel quad gpq with one 16-byte load per row; no bounds tests, no table
+  floatx4 greg[GR];
+  auto load_g_row = [&](int chunk, int j) __attribute__((always_inline)) {
+    const int k = min(chunk * (4 * kBKQ) + gkr + j, p.Kred - 1);   // rows past Kred meet zero weights
+    greg[j] = *reinterpret_cast<const floatx4*>(p.src + (uint32_t)(gbase + k * p.kStride));
+  };
+  auto store_g = [&](int buf) __attribute__((always_inline)) {
+    // transpose in registers: pixel e of the quad gets this thread's GR consecutive k values
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float* dst = reinterpret_cast<float*>(&Bs[buf][gkr >> 2][4 * gpq + e]) + (gkr & 3);
+      if constexpr (GR == 4) {
+        *reinterpret_cast<floatx4*>(dst) = floatx4{greg[0][e], greg[1][e], greg[2][e], greg[3][e]};
+      } else if constexpr (GR == 2) {
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<floatx2*>(dst) = floatx2{greg[0][e], greg[1][e]};
+      } else {
+        *dst = greg[0][e];
+      }
+    }
   };
 
   floatx4 areg[A_ITEMS];
@@ -223,6 +257,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   intx2 tab_e[nB];        // table entries {off, dhw} of the chunk being fetched (SGPRs)
 
   auto load_tab = [&](int chunk) __attribute__((always_inline)) {
+    if constexpr (GEMM) return;
 #pragma unroll
     for (int it = 0; it < B_ITEMS; ++it) {
       const int kq = chunk * kBKQ + bq0 + it * (kThreads / BN);
@@ -269,6 +304,28 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
 
   floatx16 acc[MT][NT];
 
+  auto load_all = [&](int chunk) __attribute__((always_inline)) {   // tab_e must hold `chunk`'s entries
+    if constexpr (GEMM) {
+#pragma unroll
+      for (int j = 0; j < GR; ++j) load_g_row(chunk, j);
+    } else {
+#pragma unroll
+      for (int e = 0; e < nB; ++e) load_b_elem(e);
+    }
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) load_a_item(chunk, it);
+  };
+  auto store_all = [&](int buf) __attribute__((always_inline)) {
+    if constexpr (GEMM) {
+      store_g(buf);
+    } else {
+#pragma unroll
+      for (int it = 0; it < B_ITEMS; ++it) store_b_item(buf, it);
+    }
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) store_a_item(buf, it);
+  };
+
   // One chunk of MFMAs (operand set `set`, read from LDS buffer `set` earlier) with the work for
   // the following chunks woven in between them, one small step per MFMA, so that it executes in
   // the shadow of the 64-cycle matrix instructions:
@@ -281,17 +338,25 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
     if constexpr (T >= 32) {
       constexpr int kStore = T - 8, kSync = T - 4;
-      static_assert(nB + A_ITEMS <= kStore && kStore + B_ITEMS + A_ITEMS - 1 <= kSync, "schedule does not fit");
+      constexpr int nL = GEMM ? GR : nB;   // load steps of the gathered operand
+      static_assert(nL + A_ITEMS <= kStore && kStore + B_ITEMS + A_ITEMS - 1 <= kSync, "schedule does not fit");
 #pragma unroll
       for (int s = 0; s < T; ++s) {
         const int kk = s / (4 * MT * NT), rem = s % (4 * MT * NT);
         const int j = rem / (MT * NT), x = (rem % (MT * NT)) / NT, y = rem % NT;
         acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[set][kk][x][j], opB[set][kk][y][j], acc[x][y], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        if (s < nB) load_b_elem(s);
-        else if (s < nB + A_ITEMS) load_a_item(nchunk, s - nB);
-        if (s >= kStore && s < kStore + B_ITEMS) store_b_item(set ^ 1, s - kStore);
-        else if (s >= kStore + B_ITEMS && s < kStore + B_ITEMS + A_ITEMS) store_a_item(set ^ 1, s - kStore - B_ITEMS);
+        if constexpr (GEMM) {
+          if (s < nL) load_g_row(nchunk, s);
+          else if (s < nL + A_ITEMS) load_a_item(nchunk, s - nL);
+          if (s == kStore) store_g(set ^ 1);
+          else if (s > kStore && s <= kStore + A_ITEMS) store_a_item(set ^ 1, s - kStore - 1);
+        } else {
+          if (s < nB) load_b_elem(s);
+          else if (s < nB + A_ITEMS) load_a_item(nchunk, s - nB);
+          if (s >= kStore && s < kStore + B_ITEMS) store_b_item(set ^ 1, s - kStore);
+          else if (s >= kStore + B_ITEMS && s < kStore + B_ITEMS + A_ITEMS) store_a_item(set ^ 1, s - kStore - B_ITEMS);
+        }
         if (s == kSync) {
           __syncthreads();
           read_ops(set ^ 1, set ^ 1);
@@ -300,10 +365,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
         __builtin_amdgcn_sched_barrier(0);
       }
     } else {
-#pragma unroll
-      for (int e = 0; e < nB; ++e) load_b_elem(e);
-#pragma unroll
-      for (int it = 0; it < A_ITEMS; ++it) load_a_item(nchunk, it);
+      load_all(nchunk);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < T; ++s) {
@@ -312,10 +374,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
         acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[set][kk][x][j], opB[set][kk][y][j], acc[x][y], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int it = 0; it < B_ITEMS; ++it) store_b_item(set ^ 1, it);
-#pragma unroll
-      for (int it = 0; it < A_ITEMS; ++it) store_a_item(set ^ 1, it);
+      store_all(set ^ 1);
       __syncthreads();
       read_ops(set ^ 1, set ^ 1);
       load_tab(nnchunk);
@@ -333,14 +392,8 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     if (c0 >= c1) return;
     const int last = c1 - 1;
     load_tab(c0);
-#pragma unroll
-    for (int e = 0; e < nB; ++e) load_b_elem(e);
-#pragma unroll
-    for (int it = 0; it < A_ITEMS; ++it) load_a_item(c0, it);
-#pragma unroll
-    for (int it = 0; it < B_ITEMS; ++it) store_b_item(0, it);
-#pragma unroll
-    for (int it = 0; it < A_ITEMS; ++it) store_a_item(0, it);
+    load_all(c0);
+    store_all(0);
     __syncthreads();
     read_ops(0, 0);
     load_tab(min(c0 + 1, last));
@@ -560,11 +613,14 @@ size_t sk_workspace_bytes() { return (size_t)2 * kSkBlocks * 128 * 128 * sizeof(
 
 template <int WM, int WN, int MT, int NT>
 void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+  const bool gemm = p.kStride > 0;
   if (sk_blocks > 0) {
-    igemm_f32<WM, WN, MT, NT, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    if (gemm) igemm_f32<WM, WN, MT, NT, true, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    else igemm_f32<WM, WN, MT, NT, true, false><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     igemm_fixup<WM, WN, MT, NT><<<p.tiles - p.skDpTiles, kThreads, 0, st>>>(p);
   } else {
-    igemm_f32<WM, WN, MT, NT, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+    if (gemm) igemm_f32<WM, WN, MT, NT, false, true><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+    else igemm_f32<WM, WN, MT, NT, false, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
 }
 
@@ -663,6 +719,10 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   p.srcStrideN = C * H * W; p.srcStrideG = Cg * H * W;
   p.outStrideN = K * P * Q; p.outStrideG = Kg * P * Q; p.outStrideI = P * Q; p.outRow = Q;
   p.ou = 1; p.ouh = 0; p.ov = 1; p.ovw = 0;
+  if (R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && (H * W) % 4 == 0) {
+    p.kStride = H * W;   // y[k][n,hw] = sum_c w[k][c] * x[n][c][hw]: the gathered operand is x itself
+    p.Kred = Kred;
+  }
   return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes + tab_bytes));
 }
 
@@ -791,6 +851,11 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       p.srcStrideN = K * P * Q; p.srcStrideG = Kg * P * Q;
       p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
       p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
+      if (R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && Hx == P && Wx == Q && (P * Q) % 4 == 0 &&
+          KQ > 0) {
+        p.kStride = P * Q;   // dx[c][n,hw] = sum_k w[k][c] * dy[n][k][hw]
+        p.Kred = Kred;
+      }
       if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
     }
   }

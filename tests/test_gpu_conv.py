@@ -72,6 +72,9 @@ TILE_CASES = [
     (8, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # 49 tiles of 128x128: split reduction (stream-K)
     (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # 196 tiles of 64x256: stream-K
     (8, 256, 14, 14, 256, 3, 3, (2, 2), (1, 1), (1, 1), 1),     # stream-K in every dgrad parity class
+    (2, 40, 8, 8, 72, 1, 1, (1, 1), (0, 0), (1, 1), 1),         # plain-GEMM path, 64x64 tiles, C not a multiple of 16
+    (16, 256, 14, 14, 1024, 1, 1, (1, 1), (0, 0), (1, 1), 1),   # plain-GEMM path with split left-over tiles
+    (3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2),         # plain-GEMM path with groups, ragged pixel tile
 ]
 
 
