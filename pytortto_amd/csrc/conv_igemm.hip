@@ -19,6 +19,8 @@
 // written to LDS in the same layout, so every MFMA operand fetch is one ds_read_b128 that
 // yields four k-steps.  Global loads for chunk c+1 are issued before the MFMAs of chunk c
 // (register prefetch) and land in the other LDS buffer: one barrier per chunk.
+#include <cstdlib>
+
 #include "tt_common.h"
 
 namespace {
@@ -520,16 +522,18 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   }
 }
 
-// Stream-K second stage: one block per tile; tiles that a single block computed are already
-// stored, the others are the sum of their segments' partial accumulators (added in block
-// order, so the result does not depend on timing), plus bias.
+// Stream-K second stage: MT*NT blocks per left-over tile, one per 32x32 accumulator tile of
+// each wave (more, smaller blocks: the kernel is pure latency-bound streaming).  Tiles that a
+// single block computed are already stored; the others are the sum of their segments' partial
+// accumulators (added in block order, so the result does not depend on timing), plus bias.
 template <int WM, int WN, int MT, int NT>
 __global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p) {
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int kAccQ = MT * NT * 4;
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = tid >> 6, wm = wave / WN, wn = wave % WN;
-  const int tile = p.skDpTiles + blockIdx.x;   // one block per left-over tile
+  const int tile = p.skDpTiles + blockIdx.x;
+  const int xy = blockIdx.y, x = xy / NT, y = xy % NT;
   const int nblk = p.skBlocks;
   const int chunks = p.KQ / kBKQ;
   const long long t0 = (long long)blockIdx.x * chunks, t1 = t0 + chunks;
@@ -537,32 +541,28 @@ __global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p) {
   const int b_first = (int)(((t0 + 1) * nblk - 1) / p.skIters);
   const int b_last = (int)((t1 * nblk - 1) / p.skIters);
   if (b_first == b_last) return;
-  floatx4 acc[kAccQ];
+  floatx4 acc[4];
 #pragma unroll
-  for (int q = 0; q < kAccQ; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
   for (int b = b_first; b <= b_last; ++b) {
     const long long begin = (long long)b * p.skIters / nblk;
-    const floatx4* __restrict__ src = p.skPartial + ((size_t)(2 * b + (begin > t0 ? 0 : 1)) * kAccQ) * kThreads + tid;
+    const floatx4* __restrict__ src =
+        p.skPartial + ((size_t)(2 * b + (begin > t0 ? 0 : 1)) * kAccQ + xy * 4) * kThreads + tid;
 #pragma unroll
-    for (int q = 0; q < kAccQ; ++q) acc[q] += src[(size_t)q * kThreads];
+    for (int q = 0; q < 4; ++q) acc[q] += __builtin_nontemporal_load(&src[(size_t)q * kThreads]);
   }
   const int i0 = (tile % p.tilesI) * BM, m0 = (tile / p.tilesI) * BN;
+  const int m = m0 + (wn * NT + y) * 32 + l32;
+  if (m >= p.M) return;
+  const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
+  const uint32_t rem = (uint32_t)m - n * p.divUV.d;
+  const uint32_t u = tt::fd_div(rem, p.divV);
+  const uint32_t v = rem - u * p.divV.d;
+  const uint32_t obase = (uint32_t)((int)n * p.outStrideN + ((int)u * p.ou + p.ouh) * p.outRow + (int)v * p.ov + p.ovw);
 #pragma unroll
-  for (int y = 0; y < NT; ++y) {
-    const int m = m0 + (wn * NT + y) * 32 + l32;
-    if (m >= p.M) continue;
-    const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
-    const uint32_t rem = (uint32_t)m - n * p.divUV.d;
-    const uint32_t u = tt::fd_div(rem, p.divV);
-    const uint32_t v = rem - u * p.divV.d;
-    const uint32_t obase = (uint32_t)((int)n * p.outStrideN + ((int)u * p.ou + p.ouh) * p.outRow + (int)v * p.ov + p.ovw);
-#pragma unroll
-    for (int x = 0; x < MT; ++x)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-        if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[(x * NT + y) * 4 + (r >> 2)][r & 3] + (p.bias ? p.bias[i] : 0.f);
-      }
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+    if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[r >> 2][r & 3] + (p.bias ? p.bias[i] : 0.f);
   }
 }
 
@@ -595,6 +595,10 @@ TileChoice choose_tile(int I, int M, int groups, int chunks) {
   TileChoice t;
   t.bm = I <= 64 ? 64 : 128;
   t.bn = I <= 64 ? 256 : 128;
+  if (const char* e = getenv("TT_IGEMM_TILE")) {   // tuning knob: 0 = 128x128, 1 = 64x256
+    if (e[0] == '0') { t.bm = 128; t.bn = 128; }
+    if (e[0] == '1') { t.bm = 64; t.bn = 256; }
+  }
   t.sk_blocks = 0;
   const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
   if (wants_stream_k(tiles, chunks, groups)) {
@@ -617,7 +621,7 @@ void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   if (sk_blocks > 0) {
     if (gemm) igemm_f32<WM, WN, MT, NT, true, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     else igemm_f32<WM, WN, MT, NT, true, false><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
-    igemm_fixup<WM, WN, MT, NT><<<p.tiles - p.skDpTiles, kThreads, 0, st>>>(p);
+    igemm_fixup<WM, WN, MT, NT><<<dim3(p.tiles - p.skDpTiles, MT * NT), kThreads, 0, st>>>(p);
   } else {
     if (gemm) igemm_f32<WM, WN, MT, NT, false, true><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
     else igemm_f32<WM, WN, MT, NT, false, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
