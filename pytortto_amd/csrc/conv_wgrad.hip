@@ -45,8 +45,8 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ROWS = BM / 8, B_ROWS = BN / 8;   // rows per thread (8 row groups of 32 lanes)
-  __shared__ __attribute__((aligned(16))) float As[BM][kLd];
-  __shared__ __attribute__((aligned(16))) float Bs[BN][kLd];
+  __shared__ __attribute__((aligned(16))) float As[2][BM][kLd];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BN][kLd];
   __shared__ int2 jtab[BN];   // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
@@ -74,38 +74,40 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
   const float* __restrict__ dyg = p.dy + (size_t)g * p.dyStrideG;
   const float* __restrict__ xg = p.x + (size_t)g * p.xStrideG;
 
+  // staging registers of the chunk being fetched, and what its loads need
   float areg[A_ROWS], breg[B_ROWS];
-  bool aok = false;
-  uint32_t bok = 0;   // bit t: breg[t] is inside the image (applied when written to LDS)
+  int amask = 0;        // all ones if this thread's pixel is inside the reduction range
+  uint32_t bok = 0;     // bit t: breg[t] is inside the image (applied when written to LDS)
   int2 jreg[B_ROWS];
+  int ih0 = kInvalid, iw0 = 0, xbase = 0, dybase = 0, alim = 0;
+  const int arow = i0 + rg;
 
   const int c_begin = split * p.chunksPerSplit;
   const int c_end = min(p.chunks, c_begin + p.chunksPerSplit);
 
-  auto load_global = [&](int chunk) {
+  auto decompose = [&](int chunk) __attribute__((always_inline)) {
     const int m = chunk * kBK + px;
-    int ih0 = kInvalid, iw0 = 0, xbase = 0, dybase = 0;
     const bool mok = m < p.M;
-    aok = mok;
+    const uint32_t mm = mok ? (uint32_t)m : 0u;
+    const uint32_t n = tt::fd_div(mm, p.divPQ);
+    const uint32_t pq = mm - n * p.divPQ.d;
+    const uint32_t pp = tt::fd_div(pq, p.divQ);
+    const uint32_t qq = pq - pp * p.divQ.d;
+    ih0 = mok ? (int)pp * p.sh - p.ph : kInvalid;
+    iw0 = (int)qq * p.sw - p.pw;
+    xbase = (int)n * p.xStrideN + ((int)pp * p.sh - p.ph) * p.W + iw0;
+    dybase = (int)n * p.dyStrideN + (int)pq + arow * p.PQ;
+    amask = mok ? -1 : 0;
+    alim = mok ? p.Kg : 0;   // rows at or beyond it are not read (they are never stored either)
     bok = 0;
-    if (mok) {
-      const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
-      const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
-      const uint32_t pp = tt::fd_div(pq, p.divQ);
-      const uint32_t qq = pq - pp * p.divQ.d;
-      ih0 = (int)pp * p.sh - p.ph;
-      iw0 = (int)qq * p.sw - p.pw;
-      xbase = (int)n * p.xStrideN + ih0 * p.W + iw0;
-      dybase = (int)n * p.dyStrideN + (int)pq;
-    }
-#pragma unroll
-    for (int t = 0; t < A_ROWS; ++t) {
-      const int i = i0 + rg + 8 * t;
-      const bool ok = mok && i < p.Kg;
-      areg[t] = dyg[ok ? (uint32_t)(dybase + i * p.PQ) : 0u];
-    }
-#pragma unroll
-    for (int t = 0; t < B_ROWS; ++t) {
+  };
+  auto load_step = [&](int li) __attribute__((always_inline)) {
+    if (li < A_ROWS) {
+      const int t = li;
+      const bool ok = arow + 8 * t < alim;
+      areg[t] = dyg[ok ? (uint32_t)(dybase + 8 * t * p.PQ) : 0u];
+    } else {
+      const int t = li - A_ROWS;
       const int2 e = jreg[t];
       const int ih = ih0 + (int)(short)(e.y & 0xffff);
       const int iw = iw0 + (e.y >> 16);
@@ -114,16 +116,15 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
       bok |= ok ? (1u << t) : 0u;
     }
   };
-  auto store_lds = [&]() {
-    // rows beyond Kg / columns beyond J may hold anything (never stored); pixels beyond M and
-    // taps outside the image must be exactly zero: AND with an all-ones / all-zeros word
-    const int amask = aok ? -1 : 0;
-#pragma unroll
-    for (int t = 0; t < A_ROWS; ++t) As[rg + 8 * t][px] = __int_as_float(__float_as_int(areg[t]) & amask);
-#pragma unroll
-    for (int t = 0; t < B_ROWS; ++t) {
+  // Rows beyond Kg / columns beyond J may hold anything (never stored); pixels beyond M and taps
+  // outside the image must be exactly zero: AND with an all-ones / all-zeros word.
+  auto store_step = [&](int buf, int li) __attribute__((always_inline)) {
+    if (li < A_ROWS) {
+      As[buf][rg + 8 * li][px] = __int_as_float(__float_as_int(areg[li]) & amask);
+    } else {
+      const int t = li - A_ROWS;
       const int bmask = ((int)(bok << (31 - t))) >> 31;
-      Bs[rg + 8 * t][px] = __int_as_float(__float_as_int(breg[t]) & bmask);
+      Bs[buf][rg + 8 * t][px] = __int_as_float(__float_as_int(breg[t]) & bmask);
     }
   };
 
@@ -135,37 +136,76 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  // MFMA operands of one eighth-of-a-chunk (8 pixels): two register sets, the next one is read
+  // from LDS while the current one is consumed
+  floatx4 opA[2][MT], opB[2][NT];
+  auto read_ops = [&](int set, int buf, int kk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int xx = 0; xx < MT; ++xx)
+      opA[set][xx] = *reinterpret_cast<const floatx4*>(&As[buf][(wm * MT + xx) * 32 + l32][kk * 8 + 4 * h]);
+#pragma unroll
+    for (int yy = 0; yy < NT; ++yy)
+      opB[set][yy] = *reinterpret_cast<const floatx4*>(&Bs[buf][(wn * NT + yy) * 32 + l32][kk * 8 + 4 * h]);
+  };
+
+  // One chunk (32 pixels of the reduction) of MFMAs out of LDS buffer `buf`, with the next
+  // chunk's work woven in between them, one small step per MFMA, so that it runs in the shadow
+  // of the 64-cycle matrix instructions: pixel decomposition and global loads in the first half,
+  // masked LDS writes into the other buffer from 5/8 on, then the one barrier and the first
+  // operand fetch of the next chunk.  sched_barrier pins the order.
+  constexpr int T = 16 * MT * NT;            // MFMAs per chunk
+  constexpr int PK = 4 * MT * NT;            // MFMAs per 8-pixel operand set
+  constexpr int L = A_ROWS + B_ROWS;         // loads (and LDS writes) per thread per chunk
+  constexpr int LPS = (L + T / 2 - 2) / (T / 2 - 1);       // loads per slot, slots 1 .. T/2-1
+  constexpr int kStore = 5 * T / 8, kSync = T - 4;
+  constexpr int SPS = (L + (kSync - kStore) - 1) / (kSync - kStore);   // LDS writes per slot
+  auto chunk_body = [&](const int buf, const int nchunk) __attribute__((always_inline)) {
+#pragma unroll
+    for (int s = 0; s < T; ++s) {
+      const int kk = s / PK, rem = s % PK;
+      const int j = rem / (MT * NT), xx = (rem % (MT * NT)) / NT, yy = rem % NT;
+      acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[kk & 1][xx][j], opB[kk & 1][yy][j], acc[xx][yy], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (rem == 0 && kk < 3) read_ops((kk + 1) & 1, buf, kk + 1);
+      if (s == 0) decompose(nchunk);
+#pragma unroll
+      for (int u = 0; u < LPS; ++u) {
+        const int li = (s - 1) * LPS + u;
+        if (s >= 1 && li < L) load_step(li);
+      }
+#pragma unroll
+      for (int u = 0; u < SPS; ++u) {
+        const int li = (s - kStore) * SPS + u;
+        if (s >= kStore && s < kSync && li < L) store_step(buf ^ 1, li);
+      }
+      if (s == kSync) {
+        __syncthreads();
+        read_ops(0, buf ^ 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
   __syncthreads();   // jtab
 #pragma unroll
   for (int t = 0; t < B_ROWS; ++t) jreg[t] = jtab[rg + 8 * t];
 
-  if (c_begin < c_end) load_global(c_begin);
-  for (int c = c_begin; c < c_end; ++c) {
-    store_lds();
+  if (c_begin < c_end) {
+    const int last = c_end - 1;
+    decompose(c_begin);
+#pragma unroll
+    for (int li = 0; li < L; ++li) load_step(li);
+#pragma unroll
+    for (int li = 0; li < L; ++li) store_step(0, li);
     __syncthreads();
-    load_global(min(c + 1, c_end - 1));   // in flight while the MFMAs below run (last: harmless re-fetch)
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int kk = 0; kk < kBK / 8; ++kk) {
-      floatx4 a[MT], b[NT];
-#pragma unroll
-      for (int xx = 0; xx < MT; ++xx)
-        a[xx] = *reinterpret_cast<const floatx4*>(&As[(wm * MT + xx) * 32 + l32][kk * 8 + 4 * h]);
-#pragma unroll
-      for (int yy = 0; yy < NT; ++yy)
-        b[yy] = *reinterpret_cast<const floatx4*>(&Bs[(wn * NT + yy) * 32 + l32][kk * 8 + 4 * h]);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int xx = 0; xx < MT; ++xx)
-#pragma unroll
-          for (int yy = 0; yy < NT; ++yy) {
-            acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[xx][j], b[yy][j], acc[xx][yy], 0, 0, 0);
-          }
-      }
+    read_ops(0, 0, 0);
+    // past the end the last chunk is fetched again (cache hits) instead of branching
+    int c = c_begin;
+    for (; c + 1 < c_end; c += 2) {
+      chunk_body(0, c + 1);
+      chunk_body(1, min(c + 2, last));
     }
-    __builtin_amdgcn_sched_barrier(0);
-    __syncthreads();   // every wave is done reading before the next chunk overwrites the tiles
+    if (c < c_end) chunk_body(0, last);
   }
 
   float* __restrict__ out = p.out + (size_t)split * p.outStrideSplit + (size_t)g * p.Kg * p.J;
