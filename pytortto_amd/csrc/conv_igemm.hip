@@ -20,6 +20,7 @@
 // yields four k-steps.  Global loads for chunk c+1 are issued before the MFMAs of chunk c
 // (register prefetch) and land in the other LDS buffer: one barrier per chunk.
 #include <cstdlib>
+#include <map>
 
 #include "tt_common.h"
 
@@ -56,6 +57,10 @@ struct Igemm {
   int ou, ouh, ov, ovw;      // output row = u*ou + ouh, column = v*ov + ovw
   int tilesI;                // row tiles per group
   int tiles;                 // tilesI * pixel tiles
+  // forward launches whose weight rows are a multiple of 4 long read the weights in place (a
+  // row of w is already k-major): row stride in floats, 0 = use the repacked copy in wp
+  const float* wraw;
+  int wRowStride;
   // plain-GEMM launches only (1x1, stride 1, no padding: the gathered operand is the [k][pixel]
   // matrix itself): elements between consecutive k rows, and the real reduction length
   int kStride, Kred;
@@ -204,6 +209,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   const int gpq = tid % GPQ, gkr = (tid / GPQ) * GR;
   int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0, gbase = 0;
   const floatx4* __restrict__ wsrc = p.wp;
+  const float* __restrict__ wrow = p.wraw;
   auto set_tile = [&](int tile) __attribute__((always_inline)) {
     i0 = (tile % p.tilesI) * BM;
     m0 = (tile / p.tilesI) * BN;
@@ -221,6 +227,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
     }
     wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
+    if (p.wRowStride) wrow = p.wraw + (size_t)(g * p.I + min(i0 + arow, p.I - 1)) * p.wRowStride;   // rows past I: never stored
     if constexpr (GEMM) {
       // four consecutive pixels per thread: m % 4 == 0 and (U*V) % 4 == 0, so they share n
       const int mq = min(m0 + 4 * gpq, p.M - 4);   // past-the-end quads re-read the last one; never stored
@@ -269,7 +276,13 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   };
   auto load_a_item = [&](int chunk, int it) __attribute__((always_inline)) {
     const int q = aq0 + it * (kThreads / BM);   // always < kBKQ unless the tile has fewer than 64 rows
-    if (q < kBKQ) areg[it] = wsrc[(size_t)(chunk * kBKQ + q) * p.Ipad + arow];
+    if (q < kBKQ) {
+      const int kq = chunk * kBKQ + q;
+      if (p.wRowStride)   // in place; quads past the end of the row must be zero, not garbage
+        areg[it] = 4 * kq < p.wRowStride ? *reinterpret_cast<const floatx4*>(wrow + 4 * kq) : floatx4{0.f, 0.f, 0.f, 0.f};
+      else
+        areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
+    }
   };
   auto load_b_elem = [&](int e) __attribute__((always_inline)) {   // uses tab_e: must follow load_tab() of the same chunk
     const intx2 t = tab_e[e];
@@ -660,6 +673,35 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
   return 0;
 }
 
+// Reduction-index tables depend only on the layer geometry: keep them across calls.
+struct KTabKey {
+  int v[9];
+  bool operator<(const KTabKey& o) const {
+    for (int i = 0; i < 9; ++i)
+      if (v[i] != o.v[i]) return v[i] < o.v[i];
+    return false;
+  }
+};
+__global__ void build_ktab(KEntry* __restrict__ tab, KTabArgs a) {
+  const int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < a.Kpad) write_ktab_entry(tab, a, k);
+}
+int cached_ktab(const KTabArgs& a, KEntry** out) {
+  static std::map<KTabKey, KEntry*> cache;
+  const KTabKey key{{a.Kred, a.Kpad, a.TB, a.TC, a.sa, a.sb, a.sc, a.stepH, a.stepW}};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    TT_REQUIRE(cache.size() < 4096, "too many distinct convolution geometries for the table cache");
+    KEntry* tab = nullptr;
+    TT_HIP(hipMalloc((void**)&tab, sizeof(KEntry) * (size_t)a.Kpad));
+    build_ktab<<<ceil_div(a.Kpad, 256), 256, 0, tt::stream()>>>(tab, a);
+    TT_LAUNCH_CHECK();
+    it = cache.emplace(key, tab).first;
+  }
+  *out = it->second;
+  return 0;
+}
+
 int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
                  int dh, int dw, int groups, int P, int Q) {
   TT_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0, "%s: sizes must be positive", fn);
@@ -706,15 +748,24 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   floatx4* wp = (floatx4*)ws;
   KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
   hipStream_t st = tt::stream();
+  const bool in_place = Kred % 4 == 0;   // weight rows are 16-byte aligned k-major quads already
   {
     tt::ProfScope prof(TT_PROF_CONV_PREP);
     KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
-    pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
-    TT_LAUNCH_CHECK();
+    if (in_place) {
+      if (cached_ktab(ka, &tab)) return -1;
+    } else {
+      pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
+      TT_LAUNCH_CHECK();
+    }
   }
 
   Igemm p{};
   p.src = x; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = y;
+  if (in_place) {
+    p.wraw = w;
+    p.wRowStride = Kred;
+  }
   p.I = Kg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
   p.divUV = tt::make_fastdiv((uint32_t)(P * Q));
   p.divV = tt::make_fastdiv((uint32_t)Q);
@@ -814,6 +865,27 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
   if (tt::workspace((wp_bytes + tab_bytes) * classes + sk_workspace_bytes(), &ws)) return -1;
   floatx4* sk_partial = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * classes);
 
+  // Parity classes without a tap hold only bias (or zero).  Without a bias it is cheaper to
+  // clear dx once with a streaming fill than to launch a strided store kernel per empty class.
+  bool prefilled = false;
+  if (bias == nullptr) {
+    bool any_empty = false;
+    for (int ch = 0; ch < sh && ch < Hx; ++ch) {
+      bool has = false;
+      for (int r = 0; r < R; ++r) has |= ((ch + ph - r * dh) % sh + sh) % sh == 0;
+      any_empty |= !has;
+    }
+    for (int cw = 0; cw < sw && cw < Wx; ++cw) {
+      bool has = false;
+      for (int s2 = 0; s2 < S; ++s2) has |= ((cw + pw - s2 * dw) % sw + sw) % sw == 0;
+      any_empty |= !has;
+    }
+    if (any_empty) {
+      TT_HIP(hipMemsetAsync(dx, 0, sizeof(float) * (size_t)N * C * Hx * Wx, st));
+      prefilled = true;
+    }
+  }
+
   int slot = 0;
   for (int ch = 0; ch < sh && ch < Hx; ++ch) {
     // taps r with (ch + ph - r*dh) % sh == 0
@@ -829,6 +901,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       const int nTs = s0 < 0 ? 0 : ceil_div(S - s0, sstep);
       const int V = ceil_div(Wx - cw, sw);
       const int Kred = Kg * nTr * nTs;
+      if (Kred == 0 && prefilled) continue;
       const int M = N * U * V;
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
       const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ);
