@@ -19,6 +19,13 @@
 // written to LDS in the same layout, so every MFMA operand fetch is one ds_read_b128 that
 // yields four k-steps.  Global loads for chunk c+1 are issued before the MFMAs of chunk c
 // (register prefetch) and land in the other LDS buffer: one barrier per chunk.
+//
+// Vector-ALU instructions are not free next to MFMAs on this part (measured: every VALU
+// instruction in the loop costs matrix-pipe time), so the loop keeps them to a minimum:
+// operands are fetched with buffer loads whose per-lane offset is fixed for a whole tile, the
+// reduction index only moves a scalar offset, and padding is left to the buffer range check
+// (a lane whose tap falls outside the image gets bit 31 of its offset set, two VALU
+// instructions per element, and reads 0).
 #include <cstdlib>
 #include <map>
 
@@ -35,8 +42,8 @@ constexpr int kInvalid = -(1 << 20);
 
 // One entry per reduction index k (padded with never-valid entries to a whole chunk).
 struct KEntry {
-  int off;   // element offset added to the pixel's base offset
-  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit
+  int off;   // element offset added to the pixel's base offset (tap-mask tables: byte offset, biased to be >= 0)
+  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit (tap-mask tables: tap number, 31 = padding)
 };
 
 typedef int intx2 __attribute__((ext_vector_type(2)));
@@ -61,9 +68,20 @@ struct Igemm {
   // row of w is already k-major): row stride in floats, 0 = use the repacked copy in wp
   const float* wraw;
   int wRowStride;
-  // plain-GEMM launches only (1x1, stride 1, no padding: the gathered operand is the [k][pixel]
-  // matrix itself): elements between consecutive k rows, and the real reduction length
+  // How the gathered operand is addressed:
+  //   kModeCompare: 64-bit addresses, bounds compared per element (any geometry, any size)
+  //   kModeGemm   : 1x1, stride 1, no padding: the operand is the [k][pixel] matrix of each image
+  //                 itself; 16-byte buffer loads along pixels, kStride elements between k rows
+  //   kModeTapMask: buffer loads; per tile every lane keeps one bit per tap (TB x TC <= 31 taps)
+  //                 telling whether that tap falls outside the image for its pixel
+  // The two buffer modes address relative to the first image of the tile with 32-bit byte
+  // offsets; the host selects them only when those stay below 2 GiB.
+  int mode;
   int kStride, Kred;
+  int TB, TC, stepH, stepW;  // tap window and steps of the table (tap-mask mode)
+  int voffBias;              // elements added to every lane offset so that it is never negative
+  long long srdBias;         // elements subtracted from the buffer base to make up for all biases
+  const void* wbuf;          // buffer modes: base of the weight operand (wp or wraw)
   // dense input-gradient launches only (all stride-parity classes as rows of one GEMM):
   // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
   const int4* rowtab;
@@ -80,6 +98,8 @@ struct Igemm {
 // k -> {offset, steps}.  k = (a*TB + b)*TC + c:  off = a*sa + b*sb + c*sc, steps (b*stepH, c*stepW).
 struct KTabArgs {
   int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
+  int tapMask;   // 1: entries are {4*(off + offBias), tap number b*TC + c}
+  int offBias;
 };
 __device__ __forceinline__ void write_ktab_entry(KEntry* __restrict__ tab, const KTabArgs& a, int k) {
   KEntry e;
@@ -88,9 +108,13 @@ __device__ __forceinline__ void write_ktab_entry(KEntry* __restrict__ tab, const
     const int b = t % a.TB, aa = t / a.TB;
     e.off = aa * a.sa + b * a.sb + c * a.sc;
     e.dhw = ((b * a.stepH) & 0xffff) | ((c * a.stepW) << 16);
+    if (a.tapMask) {
+      e.off = 4 * (e.off + a.offBias);
+      e.dhw = b * a.TC + c;
+    }
   } else {
     e.off = 0;
-    e.dhw = (-16384) & 0xffff;   // row far above the image: never valid
+    e.dhw = a.tapMask ? 31 : (-16384) & 0xffff;   // tap 31 / a row far above the image: never valid
   }
   tab[k] = e;
 }
@@ -185,9 +209,16 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
 }
 
-template <int WM, int WN, int MT, int NT, bool SK, bool GEMM>
+constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2;
+constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format
+constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out of range and read 0
+
+__device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
+
+template <int WM, int WN, int MT, int NT, bool SK, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   static_assert(WM * WN == 4, "four waves per block");
+  constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ITEMS = (kBKQ * BM + kThreads - 1) / kThreads, B_ITEMS = kBKQ * BN / kThreads;
   static_assert(B_ITEMS >= 1 && kThreads % BM == 0 && kThreads % BN == 0, "tile shape");
@@ -207,41 +238,79 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   const ConstKTab ktab = (ConstKTab)(uintptr_t)p.ktab;
   constexpr int GPQ = BN / 4, GR = BN / 64;
   const int gpq = tid % GPQ, gkr = (tid / GPQ) * GR;
-  int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0, gbase = 0;
+  int i0 = 0, m0 = 0, ih0 = kInvalid, iw0 = 0, base = 0;
   const floatx4* __restrict__ wsrc = p.wp;
   const float* __restrict__ wrow = p.wraw;
+  // buffer modes: resource descriptors (scalar), per-lane byte offsets fixed for the tile, and
+  // the scalar byte offset of the tile's weight rows
+  __amdgpu_buffer_rsrc_t srcSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.src, 0, kSrdRecords, kSrdFlags);
+  const __amdgpu_buffer_rsrc_t wSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.wbuf, 0, kSrdRecords, kSrdFlags);
+  int bvoff = 0, avoff = 0, asoff = 0;
+  uint32_t nmask = 0xffffffffu;   // bit t set: tap t lies outside the image for this lane's pixel
+  constexpr int AQ = kThreads / BM;   // k-quads between a thread's weight items
   auto set_tile = [&](int tile) __attribute__((always_inline)) {
     i0 = (tile % p.tilesI) * BM;
     m0 = (tile / p.tilesI) * BN;
-    ih0 = kInvalid;
-    iw0 = 0;
-    base = 0;
-    const int m = m0 + pix;
-    if (m < p.M) {
-      const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
-      const uint32_t rem = (uint32_t)m - n * p.divUV.d;
-      const uint32_t u = tt::fd_div(rem, p.divV);
-      const uint32_t v = rem - u * p.divV.d;
-      ih0 = (int)u * p.su + p.bh;
-      iw0 = (int)v * p.sv + p.bw;
-      base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
-    }
-    wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
-    if (p.wRowStride) wrow = p.wraw + (size_t)(g * p.I + min(i0 + arow, p.I - 1)) * p.wRowStride;   // rows past I: never stored
-    if constexpr (GEMM) {
-      // four consecutive pixels per thread: m % 4 == 0 and (U*V) % 4 == 0, so they share n
-      const int mq = min(m0 + 4 * gpq, p.M - 4);   // past-the-end quads re-read the last one; never stored
-      const uint32_t n = tt::fd_div((uint32_t)mq, p.divUV);
-      gbase = (int)n * p.srcStrideN + g * p.srcStrideG + (int)((uint32_t)mq - n * p.divUV.d);
+    if constexpr (BUF) {
+      const uint32_t n0 = tt::fd_div((uint32_t)__builtin_amdgcn_readfirstlane(m0), p.divUV);   // first image of the tile
+      const long long rebase = (long long)n0 * p.srcStrideN + (long long)g * p.srcStrideG - p.srdBias;
+      srcSrd = __builtin_amdgcn_make_buffer_rsrc((void*)(p.src + rebase), 0, kSrdRecords, kSrdFlags);
+      if constexpr (GEMM) {
+        // four consecutive pixels per thread: m % 4 == 0 and (U*V) % 4 == 0, so they share n
+        const int mq = min(m0 + 4 * gpq, p.M - 4);   // past-the-end quads re-read the last one; never stored
+        const uint32_t n = tt::fd_div((uint32_t)mq, p.divUV);
+        bvoff = 4 * ((int)(n - n0) * p.srcStrideN + (int)((uint32_t)mq - n * p.divUV.d) + gkr * p.kStride);
+      } else {
+        const int m = m0 + pix;
+        bvoff = 0;
+        nmask = 0xffffffffu;
+        if (m < p.M) {
+          const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
+          const uint32_t rem = (uint32_t)m - n * p.divUV.d;
+          const uint32_t u = tt::fd_div(rem, p.divV);
+          const uint32_t v = rem - u * p.divV.d;
+          const int ih = (int)u * p.su + p.bh, iw = (int)v * p.sv + p.bw;
+          bvoff = 4 * ((int)(n - n0) * p.srcStrideN + ih * p.srcRow + iw + p.voffBias);
+          uint32_t cols = 0, inside = 0;
+          for (int c = 0; c < p.TC; ++c) cols |= (uint32_t)((unsigned)(iw + c * p.stepW) < (unsigned)p.Wlim) << c;
+          for (int b = 0; b < p.TB; ++b)
+            if ((unsigned)(ih + b * p.stepH) < (unsigned)p.Hlim) inside |= cols << (b * p.TC);
+          nmask = ~inside;   // bit 31 (the padding entries' tap) always stays set: TB*TC <= 31
+        }
+      }
+      if (p.wRowStride) {   // in place; rows past I are never stored
+        avoff = 4 * (min(i0 + arow, p.I - 1) * p.wRowStride + 4 * aq0);
+        asoff = 4 * g * p.I * p.wRowStride;
+      } else {
+        avoff = 16 * (aq0 * p.Ipad + arow);
+        asoff = 16 * (g * p.KQ * p.Ipad + i0);
+      }
+    } else {
+      ih0 = kInvalid;
+      iw0 = 0;
+      base = 0;
+      const int m = m0 + pix;
+      if (m < p.M) {
+        const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
+        const uint32_t rem = (uint32_t)m - n * p.divUV.d;
+        const uint32_t u = tt::fd_div(rem, p.divV);
+        const uint32_t v = rem - u * p.divV.d;
+        ih0 = (int)u * p.su + p.bh;
+        iw0 = (int)v * p.sv + p.bw;
+        base = (int)n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0;
+      }
+      wsrc = p.wp + (size_t)g * p.KQ * p.Ipad + i0;
+      if (p.wRowStride) wrow = p.wraw + (size_t)(g * p.I + min(i0 + arow, p.I - 1)) * p.wRowStride;   // rows past I: never stored
     }
   };
 
   // plain-GEMM mode: thread (gpq, gkr) loads rows gkr .. gkr+GR-1 of the chunk's 16 k rows for
-  // pixel quad gpq with one 16-byte load per row; no bounds tests, no table
+  // pixel quad gpq with one 16-byte load per row; no bounds tests, no table (the reduction is a
+  // whole number of chunks in this mode), and only the scalar offset moves with k
   floatx4 greg[GR];
   auto load_g_row = [&](int chunk, int j) __attribute__((always_inline)) {
-    const int k = min(chunk * (4 * kBKQ) + gkr + j, p.Kred - 1);   // rows past Kred meet zero weights
-    greg[j] = *reinterpret_cast<const floatx4*>(p.src + (uint32_t)(gbase + k * p.kStride));
+    const int soff = 4 * (chunk * (4 * kBKQ) + j) * p.kStride;
+    greg[j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(srcSrd, bvoff, soff, 0));
   };
   auto store_g = [&](int buf) __attribute__((always_inline)) {
     // transpose in registers: pixel e of the quad gets this thread's GR consecutive k values
@@ -278,14 +347,25 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     const int q = aq0 + it * (kThreads / BM);   // always < kBKQ unless the tile has fewer than 64 rows
     if (q < kBKQ) {
       const int kq = chunk * kBKQ + q;
-      if (p.wRowStride)   // in place; quads past the end of the row must be zero, not garbage
+      if constexpr (BUF) {
+        // in place only when rows are a whole number of chunks long: nothing to zero
+        const int soff = asoff + (p.wRowStride ? 16 * (chunk * kBKQ + it * AQ) : 16 * (chunk * kBKQ + it * AQ) * p.Ipad);
+        areg[it] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(wSrd, avoff, soff, 0));
+      } else if (p.wRowStride) {   // in place; quads past the end of the row must be zero, not garbage
         areg[it] = 4 * kq < p.wRowStride ? *reinterpret_cast<const floatx4*>(wrow + 4 * kq) : floatx4{0.f, 0.f, 0.f, 0.f};
-      else
+      } else {
         areg[it] = wsrc[(size_t)kq * p.Ipad + arow];
+      }
     }
   };
   auto load_b_elem = [&](int e) __attribute__((always_inline)) {   // uses tab_e: must follow load_tab() of the same chunk
     const intx2 t = tab_e[e];
+    if constexpr (MODE == kModeTapMask) {
+      // {byte offset, tap}: shift the lane's "outside" bit for this tap into bit 31 of its offset
+      const uint32_t vo = ((nmask >> t.y) << 31) | (uint32_t)bvoff;
+      breg[e >> 2][e & 3] = as_float(__builtin_amdgcn_raw_buffer_load_b32(srcSrd, (int)vo, t.x, 0));
+      return;
+    }
     const int ih = ih0 + (int)(short)(t.y & 0xffff);
     const int iw = iw0 + (t.y >> 16);
     const bool ok = (unsigned)ih < (unsigned)p.Hlim && (unsigned)iw < (unsigned)p.Wlim;
@@ -298,9 +378,11 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     if (q < kBKQ) As[buf][q][arow] = areg[it];
   };
   auto store_b_item = [&](int buf, int it) __attribute__((always_inline)) {
-    floatx4 v;
+    floatx4 v = breg[it];
+    if constexpr (MODE == kModeCompare) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
+      for (int j = 0; j < 4; ++j) v[j] = bok[it][j] ? breg[it][j] : 0.f;
+    }
     Bs[buf][bq0 + it * (kThreads / BN)][pix] = v;
   };
 
@@ -596,6 +678,8 @@ constexpr int kSkBlocks = 2 * kCUs;   // two co-resident blocks per CU
 // tiles do not spread evenly over the CUs; it needs a reduction long enough to split.
 bool wants_stream_k(long long tiles, int chunks, int groups) {
   if (groups != 1 || chunks < 8) return false;
+  // many tiles and a short reduction: hardware block scheduling balances better than fixed rounds
+  if (tiles >= 3LL * kSkBlocks && chunks < 64) return false;
   if (tiles * chunks < 4LL * kSkBlocks) return false;
   const long long rounds = (tiles + kCUs - 1) / kCUs;
   return (double)tiles / (double)(rounds * kCUs) < 0.93;
@@ -628,16 +712,47 @@ TileChoice choose_tile(int I, int M, int groups, int chunks) {
 // bytes of stream-K partial accumulators for the largest tile: 2 slots per block
 size_t sk_workspace_bytes() { return (size_t)2 * kSkBlocks * 128 * 128 * sizeof(float); }
 
-template <int WM, int WN, int MT, int NT>
-void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
-  const bool gemm = p.kStride > 0;
+template <int WM, int WN, int MT, int NT, int MODE>
+void launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   if (sk_blocks > 0) {
-    if (gemm) igemm_f32<WM, WN, MT, NT, true, true><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
-    else igemm_f32<WM, WN, MT, NT, true, false><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    igemm_f32<WM, WN, MT, NT, true, MODE><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     igemm_fixup<WM, WN, MT, NT><<<dim3(p.tiles - p.skDpTiles, MT * NT), kThreads, 0, st>>>(p);
   } else {
-    if (gemm) igemm_f32<WM, WN, MT, NT, false, true><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
-    else igemm_f32<WM, WN, MT, NT, false, false><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+    igemm_f32<WM, WN, MT, NT, false, MODE><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+  }
+}
+template <int WM, int WN, int MT, int NT>
+void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+  if (p.mode == kModeGemm) launch_mode<WM, WN, MT, NT, kModeGemm>(p, groups, sk_blocks, st);
+  else if (p.mode == kModeTapMask) launch_mode<WM, WN, MT, NT, kModeTapMask>(p, groups, sk_blocks, st);
+  else launch_mode<WM, WN, MT, NT, kModeCompare>(p, groups, sk_blocks, st);
+}
+
+// Picks how the kernel addresses the gathered operand (see Igemm::mode) and completes the table
+// arguments accordingly.  Needs the source geometry fields of `p`; `pixels` = U*V pixels per
+// image, `gemm_geometry` = 1x1 / stride 1 / unpadded / pixel count a multiple of 4.
+void choose_mode(Igemm& p, KTabArgs& ka, bool gemm_geometry, int N, int U, int V, long long weight_bytes) {
+  p.mode = kModeCompare;
+  p.TB = ka.TB; p.TC = ka.TC; p.stepH = ka.stepH; p.stepW = ka.stepW;
+  const long long b1 = (long long)(p.bh < 0 ? -p.bh : 0) * p.srcRow + (p.bw < 0 ? -p.bw : 0);
+  const long long lo_b = (long long)(ka.TB - 1) * ka.sb, lo_c = (long long)(ka.TC - 1) * ka.sc;
+  const long long b2 = -((lo_b < 0 ? lo_b : 0) + (lo_c < 0 ? lo_c : 0));
+  // byte offsets a lane can reach: the images one 256-pixel tile spans, one more for the
+  // reduction offset, the rows and columns its taps may overshoot, and the biases
+  const long long span = (long long)(255 / ((long long)U * V) + 2 < N ? 255 / ((long long)U * V) + 2 : N);
+  const long long reach = 4 * ((span + 1) * p.srcStrideN + 2 * (b1 + b2) +
+                               ((long long)U * p.su + (p.bh < 0 ? -p.bh : p.bh) + 2) * p.srcRow + (long long)V * p.sv +
+                               (p.bw < 0 ? -p.bw : p.bw));
+  const long long limit = (1LL << 31) - (1LL << 20);
+  if (reach >= limit || weight_bytes >= limit) return;
+  if (gemm_geometry && ka.Kred % (4 * kBKQ) == 0) {
+    p.mode = kModeGemm;
+  } else if (ka.TB * ka.TC <= 31) {
+    p.mode = kModeTapMask;
+    p.voffBias = (int)b1;
+    p.srdBias = b1 + b2;
+    ka.tapMask = 1;
+    ka.offBias = (int)b2;
   }
 }
 
@@ -675,9 +790,9 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
 
 // Reduction-index tables depend only on the layer geometry: keep them across calls.
 struct KTabKey {
-  int v[9];
+  int v[11];
   bool operator<(const KTabKey& o) const {
-    for (int i = 0; i < 9; ++i)
+    for (int i = 0; i < 11; ++i)
       if (v[i] != o.v[i]) return v[i] < o.v[i];
     return false;
   }
@@ -688,7 +803,7 @@ __global__ void build_ktab(KEntry* __restrict__ tab, KTabArgs a) {
 }
 int cached_ktab(const KTabArgs& a, KEntry** out) {
   static std::map<KTabKey, KEntry*> cache;
-  const KTabKey key{{a.Kred, a.Kpad, a.TB, a.TC, a.sa, a.sb, a.sc, a.stepH, a.stepW}};
+  const KTabKey key{{a.Kred, a.Kpad, a.TB, a.TC, a.sa, a.sb, a.sc, a.stepH, a.stepW, a.tapMask, a.offBias}};
   auto it = cache.find(key);
   if (it == cache.end()) {
     TT_REQUIRE(cache.size() < 4096, "too many distinct convolution geometries for the table cache");
@@ -748,24 +863,16 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   floatx4* wp = (floatx4*)ws;
   KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
   hipStream_t st = tt::stream();
-  const bool in_place = Kred % 4 == 0;   // weight rows are 16-byte aligned k-major quads already
-  {
-    tt::ProfScope prof(TT_PROF_CONV_PREP);
-    KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw};
-    if (in_place) {
-      if (cached_ktab(ka, &tab)) return -1;
-    } else {
-      pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
-      TT_LAUNCH_CHECK();
-    }
-  }
+  // weight rows that are a whole number of chunks long are k-major 16-byte quads already
+  const bool in_place = Kred % (4 * kBKQ) == 0;
 
   Igemm p{};
-  p.src = x; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = y;
+  p.src = x; p.wp = wp; p.bias = bias; p.out = y;
   if (in_place) {
     p.wraw = w;
     p.wRowStride = Kred;
   }
+  p.wbuf = in_place ? (const void*)w : (const void*)wp;
   p.I = Kg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
   p.divUV = tt::make_fastdiv((uint32_t)(P * Q));
   p.divV = tt::make_fastdiv((uint32_t)Q);
@@ -774,10 +881,22 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   p.srcStrideN = C * H * W; p.srcStrideG = Cg * H * W;
   p.outStrideN = K * P * Q; p.outStrideG = Kg * P * Q; p.outStrideI = P * Q; p.outRow = Q;
   p.ou = 1; p.ouh = 0; p.ov = 1; p.ovw = 0;
-  if (R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && (H * W) % 4 == 0) {
-    p.kStride = H * W;   // y[k][n,hw] = sum_c w[k][c] * x[n][c][hw]: the gathered operand is x itself
-    p.Kred = Kred;
+  // y[k][n,hw] = sum_c w[k][c] * x[n][c][hw]: for 1x1 layers the gathered operand is x itself
+  p.kStride = H * W;
+  p.Kred = Kred;
+  KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw, 0, 0};
+  choose_mode(p, ka, R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && (H * W) % 4 == 0, N, P, Q,
+              in_place ? (long long)sizeof(float) * K * Kred : (long long)wp_bytes);
+  {
+    tt::ProfScope prof(TT_PROF_CONV_PREP);
+    if (in_place) {
+      if (cached_ktab(ka, &tab)) return -1;
+    } else {
+      pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
+      TT_LAUNCH_CHECK();
+    }
   }
+  p.ktab = tab;
   return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes + tab_bytes));
 }
 
@@ -833,15 +952,8 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       floatx4* wp = (floatx4*)ws;
       KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
       int4* rowtab = (int4*)((char*)ws + wp_bytes + tab_bytes);
-      {
-        tt::ProfScope prof(TT_PROF_CONV_PREP);
-        PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx};
-        KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1};
-        pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa, tab, ka, rowtab);
-        TT_LAUNCH_CHECK();
-      }
       Igemm p{};
-      p.src = dy; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.src = dy; p.wp = wp; p.wbuf = wp; p.ktab = tab; p.bias = bias; p.out = dx;
       p.I = I; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
       p.divUV = tt::make_fastdiv((uint32_t)(U * V));
       p.divV = tt::make_fastdiv((uint32_t)V);
@@ -851,6 +963,14 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       p.outStrideN = C * Hx * Wx; p.outStrideG = 0; p.outStrideI = 0; p.outRow = Wx;
       p.ou = sh; p.ouh = 0; p.ov = sw; p.ovw = 0;
       p.rowtab = rowtab; p.outH = Hx; p.outW = Wx;
+      KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1, 0, 0};
+      choose_mode(p, ka, false, N, U, V, (long long)wp_bytes);
+      {
+        tt::ProfScope prof(TT_PROF_CONV_PREP);
+        PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx};
+        pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa, tab, ka, rowtab);
+        TT_LAUNCH_CHECK();
+      }
       return launch_igemm(p, 1, t, TT_PROF_CONV_IGEMM_DGRAD, nullptr);
     }
   }
@@ -909,17 +1029,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
       Igemm p{};
-      if (KQ > 0) {
-        tt::ProfScope prof(TT_PROF_CONV_PREP);
-        PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
-        KTabArgs ka{Kred, KQ * 4, nTr, nTs, P * Q, -eh * Q, -ew, -eh, -ew};
-        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
-        TT_LAUNCH_CHECK();
-        // h = u*sh + ch reads dy row (h + ph - r0*dh)/sh = u + (ch + ph - r0*dh)/sh  (exact)
-        p.bh = (ch + ph - r0 * dh) / sh;   // numerator is a multiple of sh by choice of r0
-        p.bw = (cw + pw - s0 * dw) / sw;
-      }
-      p.src = dy; p.wp = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.src = dy; p.wp = wp; p.wbuf = wp; p.ktab = tab; p.bias = bias; p.out = dx;
       p.I = Cg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
       p.divUV = tt::make_fastdiv((uint32_t)(U * V));
       p.divV = tt::make_fastdiv((uint32_t)V);
@@ -928,10 +1038,20 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       p.srcStrideN = K * P * Q; p.srcStrideG = Kg * P * Q;
       p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
       p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
-      if (R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && Hx == P && Wx == Q && (P * Q) % 4 == 0 &&
-          KQ > 0) {
-        p.kStride = P * Q;   // dx[c][n,hw] = sum_k w[k][c] * dy[n][k][hw]
-        p.Kred = Kred;
+      p.kStride = P * Q;   // 1x1 layers: dx[c][n,hw] = sum_k w[k][c] * dy[n][k][hw]
+      p.Kred = Kred;
+      if (KQ > 0) {
+        // h = u*sh + ch reads dy row (h + ph - r0*dh)/sh = u + (ch + ph - r0*dh)/sh  (exact)
+        p.bh = (ch + ph - r0 * dh) / sh;   // numerator is a multiple of sh by choice of r0
+        p.bw = (cw + pw - s0 * dw) / sw;
+        KTabArgs ka{Kred, KQ * 4, nTr, nTs, P * Q, -eh * Q, -ew, -eh, -ew, 0, 0};
+        choose_mode(p, ka,
+                    R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && Hx == P && Wx == Q && (P * Q) % 4 == 0,
+                    N, U, V, (long long)wp_bytes);
+        tt::ProfScope prof(TT_PROF_CONV_PREP);
+        PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
+        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
+        TT_LAUNCH_CHECK();
       }
       if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
     }
