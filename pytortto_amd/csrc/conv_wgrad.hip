@@ -12,6 +12,14 @@
 // operand fetch is one ds_read_b128 holding four reduction steps, conflict-free because
 // consecutive rows start 36 floats apart.  v_mfma_f32_32x32x2_f32 rows = output channels,
 // columns = (c,r,s), so 32 lanes store 128 contiguous bytes of dw.
+//
+// Vector-ALU instructions cost matrix-pipe time on this part, so the usual launch (BUF) fetches
+// with buffer loads: per chunk a lane computes one byte offset for its pixel in dy and one in x,
+// each load adds a per-lane constant (row / column offset), padding taps set bit 31 of the
+// offset from a per-chunk tap mask and read 0 through the buffer range check, and nothing is
+// masked when the values are written to LDS.  Offsets are relative to the first image of the
+// chunk; geometries whose offsets could reach 2 GiB, or with more than 31 taps, take the
+// compare-and-select path instead.
 #include "tt_common.h"
 
 namespace {
@@ -38,16 +46,38 @@ struct Wgrad {
   int PQ;
   int tilesI;
   size_t outStrideSplit;      // G*Kg*J
+  int R, S;                   // buffer path: taps, one bit each in the per-chunk mask
+  int xBias;                  // buffer path: ph*W + pw, keeps lane offsets non-negative
+  tt::FastDiv divDh, divDw;   // buffer path: division by the dilation
+  uint32_t rowOnes;           // buffer path: bit r*S set for every tap row r
 };
 
-template <int WM, int WN, int MT, int NT>
-__global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
+constexpr int kSrdFlags = 0x00020000;     // raw buffer, 32-bit data format
+constexpr int kSrdRecords = 0x7fffffff;   // offsets with bit 31 set are out of range and read 0
+__device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
+
+// Taps t = 0..n-1 sit at pos + t*step; those with 0 <= pos + t*step < lim form a range [lo, hi].
+// Returns the bits [lo*unit, (hi+1)*unit) (n*unit <= 31), without a loop.
+__device__ __forceinline__ uint32_t tap_range_bits(int pos, int lim, int n, int unit, const tt::FastDiv& step) {
+  int lo = pos >= 0 ? 0 : (int)tt::fd_div((uint32_t)(-pos + (int)step.d - 1), step);
+  const int room = lim - 1 - pos;
+  const int hi = room < 0 ? -1 : min(n - 1, (int)tt::fd_div((uint32_t)room, step));
+  lo = min(lo, n);
+  const uint32_t upto = (1u << ((hi + 1) * unit)) - 1u, below = (1u << (lo * unit)) - 1u;
+  return lo > hi ? 0u : upto & ~below;
+}
+
+// Two blocks per CU is all the LDS tiles allow: tell the compiler not to squeeze registers (and
+// spill) for a third wave per SIMD.
+template <int WM, int WN, int MT, int NT, bool BUF>
+__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_f32(const Wgrad p) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ROWS = BM / 8, B_ROWS = BN / 8;   // rows per thread (8 row groups of 32 lanes)
   __shared__ __attribute__((aligned(16))) float As[2][BM][kLd];
   __shared__ __attribute__((aligned(16))) float Bs[2][BN][kLd];
-  __shared__ int2 jtab[BN];   // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}
+  // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}; buffer path: {4 * offset, tap r*S + s}
+  __shared__ int2 jtab[BN];
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -58,7 +88,7 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
 
   if (tid < BN) {
     const int j = j0 + tid;
-    int2 e = make_int2(0, (-16384) & 0xffff);   // column beyond J: never valid
+    int2 e = make_int2(0, BUF ? 31 : (-16384) & 0xffff);   // column beyond J: never valid
     if (j < p.J) {
       const uint32_t c = tt::fd_div((uint32_t)j, p.divRS);
       const uint32_t rs = (uint32_t)j - c * p.divRS.d;
@@ -66,6 +96,10 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
       const uint32_t s = rs - r * p.divS.d;
       e.x = (int)c * p.HW + (int)r * p.dh * p.W + (int)s * p.dw;
       e.y = (((int)r * p.dh) & 0xffff) | (((int)s * p.dw) << 16);
+      if (BUF) {
+        e.x *= 4;
+        e.y = (int)rs;
+      }
     }
     jtab[tid] = e;
   }
@@ -85,7 +119,45 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
   const int c_begin = split * p.chunksPerSplit;
   const int c_end = min(p.chunks, c_begin + p.chunksPerSplit);
 
+  // buffer path: descriptors re-based to the chunk's first image, this lane's pixel offsets in
+  // dy and x (bit 31 of the dy offset set for pixels past the end), its tap mask (bit t set: tap
+  // t is outside the image), and the per-lane constants added per load
+  __amdgpu_buffer_rsrc_t dySrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.dy, 0, kSrdRecords, kSrdFlags);
+  __amdgpu_buffer_rsrc_t xSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, kSrdRecords, kSrdFlags);
+  uint32_t dyvoff = 0x80000000u, xvoff = 0, nmask = 0xffffffffu;
+  int aoff[A_ROWS];
+  if constexpr (BUF) {
+#pragma unroll
+    for (int t = 0; t < A_ROWS; ++t) aoff[t] = 4 * min(arow + 8 * t, p.Kg - 1) * p.PQ;   // rows past Kg are never stored
+  }
+
   auto decompose = [&](int chunk) __attribute__((always_inline)) {
+    if constexpr (BUF) {
+      const int mfirst = __builtin_amdgcn_readfirstlane(chunk * kBK);
+      const uint32_t n0 = tt::fd_div((uint32_t)mfirst, p.divPQ);
+      dySrd = __builtin_amdgcn_make_buffer_rsrc((void*)(p.dy + ((size_t)n0 * p.dyStrideN + (size_t)g * p.dyStrideG)), 0,
+                                                kSrdRecords, kSrdFlags);
+      xSrd = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(p.x + ((long long)n0 * p.xStrideN + (long long)g * p.xStrideG - p.xBias)), 0, kSrdRecords, kSrdFlags);
+      const int m = chunk * kBK + px;
+      dyvoff = 0x80000000u;
+      xvoff = 0;
+      nmask = 0xffffffffu;
+      if (m < p.M) {
+        const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
+        const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
+        const uint32_t pp = tt::fd_div(pq, p.divQ);
+        const uint32_t qq = pq - pp * p.divQ.d;
+        const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
+        dyvoff = 4u * (uint32_t)((int)(n - n0) * p.dyStrideN + (int)pq);
+        xvoff = 4u * (uint32_t)((int)(n - n0) * p.xStrideN + ih * p.W + iw + p.xBias);
+        // valid tap columns, replicated into every valid tap row (fields of S bits: no carries)
+        const uint32_t cols = tap_range_bits(iw, p.W, p.S, 1, p.divDw);
+        const uint32_t rows = tap_range_bits(ih, p.H, p.R, p.S, p.divDh) & p.rowOnes;
+        nmask = ~(cols * rows);   // bit 31 (columns past J) stays set: R*S <= 31
+      }
+      return;
+    }
     const int m = chunk * kBK + px;
     const bool mok = m < p.M;
     const uint32_t mm = mok ? (uint32_t)m : 0u;
@@ -102,6 +174,17 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
     bok = 0;
   };
   auto load_step = [&](int li) __attribute__((always_inline)) {
+    if constexpr (BUF) {
+      if (li < A_ROWS) {
+        areg[li] = as_float(__builtin_amdgcn_raw_buffer_load_b32(dySrd, (int)(dyvoff + (uint32_t)aoff[li]), 0, 0));
+      } else {
+        const int t = li - A_ROWS;
+        const int2 e = jreg[t];
+        const uint32_t vo = ((nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
+        breg[t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
+      }
+      return;
+    }
     if (li < A_ROWS) {
       const int t = li;
       const bool ok = arow + 8 * t < alim;
@@ -119,6 +202,11 @@ __global__ __launch_bounds__(kThreads, 2) void wgrad_f32(const Wgrad p) {
   // Rows beyond Kg / columns beyond J may hold anything (never stored); pixels beyond M and taps
   // outside the image must be exactly zero: AND with an all-ones / all-zeros word.
   auto store_step = [&](int buf, int li) __attribute__((always_inline)) {
+    if constexpr (BUF) {   // padding and pixels past the end were read as zeros
+      if (li < A_ROWS) As[buf][rg + 8 * li][px] = areg[li];
+      else Bs[buf][rg + 8 * (li - A_ROWS)][px] = breg[li - A_ROWS];
+      return;
+    }
     if (li < A_ROWS) {
       As[buf][rg + 8 * li][px] = __int_as_float(__float_as_int(areg[li]) & amask);
     } else {
@@ -270,6 +358,12 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce(const float* __restrict
 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+template <int WM, int WN, int MT, int NT>
+void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, hipStream_t st) {
+  if (buf) wgrad_f32<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
+  else wgrad_f32<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
+}
+
 }  // namespace
 
 extern "C" {
@@ -297,8 +391,13 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   const int tilesI = ceil_div(Kg, bm), tilesJ = ceil_div(J, bn);
   const long long tiles = (long long)tilesI * tilesJ * groups;
   const int chunks = ceil_div(M, kBK);
-  // enough blocks for ~3 per CU, but at least 8 chunks (256 pixels) of work per split
-  int splits = (int)((768 + tiles - 1) / tiles);
+  // Two blocks fit a CU (LDS), so 512 run at a time and all take equally long: fill one round of
+  // 512 as well as possible, or two rounds if that fills them clearly better; at least 8 chunks
+  // (256 pixels) of work per split.
+  const int kSlots = 512;
+  int splits = (int)(kSlots / tiles);
+  const int two = (int)(2 * kSlots / tiles);
+  if ((double)tiles * two / (2.0 * kSlots) > (double)tiles * splits / kSlots + 0.08) splits = two;
   if (splits > chunks / 8) splits = chunks / 8;
   if (splits < 1) splits = 1;
   if (splits > 4096) splits = 4096;
@@ -327,18 +426,29 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   p.PQ = P * Q;
   p.tilesI = tilesI;
   p.outStrideSplit = elems;
+  p.R = R; p.S = S;
+  p.xBias = ph * W + pw;
+  p.divDh = tt::make_fastdiv((uint32_t)dh);
+  p.divDw = tt::make_fastdiv((uint32_t)dw_);
+  if (R * S <= 31)
+    for (int r = 0; r < R; ++r) p.rowOnes |= 1u << (r * S);
+  // buffer path: byte offsets relative to the first image of a 32-pixel chunk stay below 2 GiB
+  // (a chunk spans at most 33 images; x offsets also carry the column's tap and channel offset)
+  const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
+                               ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
+  const bool buf = R * S <= 31 && reach < (1LL << 31) - (1LL << 20);
   dim3 grid(tilesI * tilesJ, groups, splits);
   hipStream_t st = tt::stream();
   {
-  tt::ProfScope prof(TT_PROF_CONV_WGRAD);
-  if (bm == 128 && bn == 128)
-    wgrad_f32<2, 2, 2, 2><<<grid, kThreads, 0, st>>>(p);
-  else if (bm == 64 && bn == 128)
-    wgrad_f32<2, 2, 1, 2><<<grid, kThreads, 0, st>>>(p);
-  else if (bm == 128 && bn == 64)
-    wgrad_f32<2, 2, 2, 1><<<grid, kThreads, 0, st>>>(p);
-  else
-    wgrad_f32<2, 2, 1, 1><<<grid, kThreads, 0, st>>>(p);
+    tt::ProfScope prof(TT_PROF_CONV_WGRAD);
+    if (bm == 128 && bn == 128)
+      launch_wgrad<2, 2, 2, 2>(p, grid, buf, st);
+    else if (bm == 64 && bn == 128)
+      launch_wgrad<2, 2, 1, 2>(p, grid, buf, st);
+    else if (bm == 128 && bn == 64)
+      launch_wgrad<2, 2, 2, 1>(p, grid, buf, st);
+    else
+      launch_wgrad<2, 2, 1, 1>(p, grid, buf, st);
   }
   TT_LAUNCH_CHECK();
   if (splits > 1) {
