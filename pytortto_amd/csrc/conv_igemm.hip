@@ -582,37 +582,46 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     // back and invalidate whole L2s on this multi-die part and cost more than the second launch.)
     constexpr int kAccQ = MT * NT * 4;
     const int b = xcd_remap(blockIdx.x, gridDim.x);
-    for (int tile = b; tile < p.skDpTiles; tile += gridDim.x) {
-      set_tile(tile);
-      run_segment(0, chunks);
-      epilogue();
-      __syncthreads();   // the next tile's first stores reuse LDS buffer 0
-    }
+    // The second block that lands on each CU (block index in the upper half of the grid) does its
+    // share of the split tiles first and its whole tiles afterwards: the two blocks of a CU then
+    // reach their store phases at different times, and one block's stores overlap the other's MFMAs.
+    const bool split_first = 2 * blockIdx.x >= gridDim.x;
+    int dp_tile = b;
+    long long it = 0, end = 0;
     if (b < p.skBlocks) {
-      long long it = (long long)b * p.skIters / p.skBlocks;
-      const long long end = (long long)(b + 1) * p.skIters / p.skBlocks;
-      while (it < end) {
+      it = (long long)b * p.skIters / p.skBlocks;
+      end = (long long)(b + 1) * p.skIters / p.skBlocks;
+    }
+    for (;;) {
+      const bool has_dp = dp_tile < p.skDpTiles, has_split = it < end;
+      if (!has_dp && !has_split) break;
+      int tile, c0 = 0, n = chunks;
+      if (has_split && (split_first || !has_dp)) {
         const int t = (int)(it / chunks);
-        const int c0 = (int)(it - (long long)t * chunks);
-        const int n = (int)min((long long)(chunks - c0), end - it);
-        set_tile(p.skDpTiles + t);
-        run_segment(c0, c0 + n);
-        if (n == chunks) {
-          epilogue();
-        } else {
-          floatx4* __restrict__ dst = p.skPartial + ((size_t)(2 * b + (c0 == 0 ? 1 : 0)) * kAccQ) * kThreads + tid;
-#pragma unroll
-          for (int x = 0; x < MT; ++x)
-#pragma unroll
-            for (int y = 0; y < NT; ++y)
-#pragma unroll
-              for (int q = 0; q < 4; ++q)
-                dst[(size_t)((x * NT + y) * 4 + q) * kThreads] =
-                    floatx4{acc[x][y][4 * q], acc[x][y][4 * q + 1], acc[x][y][4 * q + 2], acc[x][y][4 * q + 3]};
-        }
+        c0 = (int)(it - (long long)t * chunks);
+        n = (int)min((long long)(chunks - c0), end - it);
+        tile = p.skDpTiles + t;
         it += n;
-        __syncthreads();
+      } else {
+        tile = dp_tile;
+        dp_tile += gridDim.x;
       }
+      set_tile(tile);
+      run_segment(c0, c0 + n);
+      if (n == chunks) {
+        epilogue();
+      } else {
+        floatx4* __restrict__ dst = p.skPartial + ((size_t)(2 * b + (c0 == 0 ? 1 : 0)) * kAccQ) * kThreads + tid;
+#pragma unroll
+        for (int x = 0; x < MT; ++x)
+#pragma unroll
+          for (int y = 0; y < NT; ++y)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              dst[(size_t)((x * NT + y) * 4 + q) * kThreads] =
+                  floatx4{acc[x][y][4 * q], acc[x][y][4 * q + 1], acc[x][y][4 * q + 2], acc[x][y][4 * q + 3]};
+      }
+      __syncthreads();   // the next segment's first stores reuse LDS buffer 0
     }
   }
 }
@@ -672,7 +681,7 @@ struct TileChoice {
 };
 
 constexpr int kCUs = 256;             // MI355X
-constexpr int kSkBlocks = 2 * kCUs;   // two co-resident blocks per CU
+constexpr int kSkBlocks = 2 * kCUs;   // persistent launches: two blocks per CU (three or four measured slower)
 
 // Stream-K pays (a second small kernel, partial tiles through HBM) and only helps when the
 // tiles do not spread evenly over the CUs; it needs a reduction long enough to split.
@@ -688,7 +697,7 @@ bool wants_stream_k(long long tiles, int chunks, int groups) {
 // 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
 // CUs idle or unevenly loaded the reduction is split stream-K fashion; if it is too short for
 // that, 64x64 tiles raise the block count instead.
-TileChoice choose_tile(int I, int M, int groups, int chunks) {
+TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k = true) {
   TileChoice t;
   t.bm = I <= 64 ? 64 : 128;
   t.bn = I <= 64 ? 256 : 128;
@@ -698,13 +707,13 @@ TileChoice choose_tile(int I, int M, int groups, int chunks) {
   }
   t.sk_blocks = 0;
   const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
-  if (wants_stream_k(tiles, chunks, groups)) {
+  if (allow_stream_k && wants_stream_k(tiles, chunks, groups)) {
     t.sk_blocks = kSkBlocks;
   } else if (tiles * groups < kCUs) {
     t.bm = 64;
     t.bn = 64;
     const long long small = (long long)ceil_div(I, 64) * ceil_div(M, 64);
-    if (wants_stream_k(small, chunks, groups)) t.sk_blocks = kSkBlocks;
+    if (allow_stream_k && wants_stream_k(small, chunks, groups)) t.sk_blocks = kSkBlocks;
   }
   return t;
 }
@@ -1006,6 +1015,17 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
     }
   }
 
+  // Several classes with taps mean several short launches in a row; a fix-up stage after each
+  // costs more than the imbalance it removes (measured on 3x3 stride-2 layers).
+  int tap_rows = 0, tap_cols = 0;
+  for (int ch = 0; ch < sh && ch < Hx; ++ch)
+    for (int r = 0; r < R; ++r)
+      if (((ch + ph - r * dh) % sh + sh) % sh == 0) { ++tap_rows; break; }
+  for (int cw = 0; cw < sw && cw < Wx; ++cw)
+    for (int s2 = 0; s2 < S; ++s2)
+      if (((cw + pw - s2 * dw) % sw + sw) % sw == 0) { ++tap_cols; break; }
+  const bool allow_stream_k = tap_rows * tap_cols <= 1;
+
   int slot = 0;
   for (int ch = 0; ch < sh && ch < Hx; ++ch) {
     // taps r with (ch + ph - r*dh) % sh == 0
@@ -1024,7 +1044,7 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       if (Kred == 0 && prefilled) continue;
       const int M = N * U * V;
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
-      const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ);
+      const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k);
       const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
