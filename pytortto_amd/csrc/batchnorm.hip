@@ -88,6 +88,8 @@ __device__ __forceinline__ void load_partials(const double2* __restrict__ partia
   b = wave_sum(p.y);
 }
 
+constexpr int kStreamU = 8;   // float4 loads in flight per thread in the stream reduce kernel
+
 struct Geometry {
   int N, C, HW;         // HW in floats
   int splits;           // gridDim.x
@@ -146,6 +148,67 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_planes(const float* __rest
             b.x = fmaf(d.x, d.x, b.x); b.y = fmaf(d.y, d.y, b.y);
             b.z = fmaf(d.z, d.z, b.z); b.w = fmaf(d.w, d.w, b.w);
           }
+        }
+      }
+    }
+    sa += ((double)a.x + (double)a.y) + ((double)a.z + (double)a.w);
+    sb += ((double)b.x + (double)b.y) + ((double)b.z + (double)b.w);
+  }
+  block_sum2(sa, sb, lds);
+  if (threadIdx.x == 0) partial[(size_t)c * g.splits + split] = make_double2(sa, sb);
+}
+
+// Stream kernel: HW % 4 == 0.  A block takes a contiguous range of the channel's N*HW/4 float4
+// vectors (flattened over planes, so no batch is cut short at a plane end) and issues kU loads
+// per tensor and thread before it consumes the first: enough bytes in flight per block that the
+// reduction tails of other blocks do not leave the memory system idle.
+template <int kKind>
+__global__ __launch_bounds__(kThreads) void bn_reduce_stream(const float* __restrict__ x,
+                                                             const float* __restrict__ dy,
+                                                             const float* __restrict__ mean,
+                                                             double2* __restrict__ partial, Geometry g) {
+  __shared__ double lds[2 * kWaves];
+  const int c = blockIdx.y, split = blockIdx.x;
+  constexpr bool kBwd = kKind == 1;
+  constexpr int kU = kBwd ? kStreamU / 2 : kStreamU;
+  const uint32_t hwv = (uint32_t)g.HW >> 2;
+  const uint32_t total = (uint32_t)g.N * hwv;
+  const float ref = kKind == 1 ? mean[c] : (kKind == 0 ? x[(size_t)c * g.HW] : 0.f);
+  const uint32_t e0 = (uint32_t)split * (uint32_t)g.per_block;
+  const uint32_t e1 = min(total, e0 + (uint32_t)g.per_block);
+  const float4 fill = make_float4(ref, ref, ref, ref);
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  double sa = 0.0, sb = 0.0;
+  for (uint32_t base = e0; base < e1; base += kThreads * kU) {
+    float4 v[kU], gq[kU];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const uint32_t e = base + threadIdx.x + kThreads * u;
+      const bool ok = e < e1;
+      const uint32_t ee = ok ? e : e0;   // past the end: re-read a valid vector, use the neutral value
+      const uint32_t n = tt::fd_div(ee, g.hwv_div);
+      const size_t off = ((size_t)n * g.C + c) * g.HW + (size_t)(ee - n * hwv) * 4;
+      const float4 t = *reinterpret_cast<const float4*>(x + off);
+      v[u] = ok ? t : fill;
+      if constexpr (kBwd) {
+        const float4 q = *reinterpret_cast<const float4*>(dy + off);
+        gq[u] = ok ? q : zero;
+      }
+    }
+    float4 a = zero, b = zero;
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      float4 d = v[u];
+      d.x -= ref; d.y -= ref; d.z -= ref; d.w -= ref;
+      if (kBwd) {
+        a.x += gq[u].x; a.y += gq[u].y; a.z += gq[u].z; a.w += gq[u].w;
+        b.x = fmaf(gq[u].x, d.x, b.x); b.y = fmaf(gq[u].y, d.y, b.y);
+        b.z = fmaf(gq[u].z, d.z, b.z); b.w = fmaf(gq[u].w, d.w, b.w);
+      } else {
+        a.x += d.x; a.y += d.y; a.z += d.z; a.w += d.w;
+        if (kKind == 0) {
+          b.x = fmaf(d.x, d.x, b.x); b.y = fmaf(d.y, d.y, b.y);
+          b.z = fmaf(d.z, d.z, b.z); b.w = fmaf(d.w, d.w, b.w);
         }
       }
     }
@@ -298,6 +361,7 @@ struct FwdArgs {
   const float* given_mean;  // eval mode: statistics are inputs, no partials
   const float* given_var;
   const double2* partial;
+  int partial_splits;       // partials per channel written by the first sweep
   float one_minus_mom, mom, unbias, eps;
 };
 
@@ -314,7 +378,7 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_apply(FwdArgs a, Geometry g) 
       var = a.given_var[c];
     } else {
       double s1, s2;
-      load_partials(a.partial, c, g.splits, s1, s2);
+      load_partials(a.partial, c, a.partial_splits, s1, s2);
       const double m = (double)g.N * (double)g.HW;
       const double shift = (double)a.x[(size_t)c * g.HW];
       const double d1 = s1 / m;
@@ -361,6 +425,7 @@ struct BwdArgs {
   float* dgamma;
   float* dbeta;
   const double2* partial;
+  int partial_splits;
 };
 
 template <int kMode>
@@ -370,7 +435,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) 
   const int split = g.splits - 1 - (int)blockIdx.x;
   if (threadIdx.x < tt::kWave) {
     double s_dy, s_dyxmu;
-    load_partials(a.partial, c, g.splits, s_dy, s_dyxmu);
+    load_partials(a.partial, c, a.partial_splits, s_dy, s_dyxmu);
     if (threadIdx.x == 0) {
       const double m = (double)g.N * (double)g.HW;
       const double sd = (double)a.save_sd[c];
@@ -399,6 +464,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 // Picks the kernel flavour and how a channel is shared between blocks.
+constexpr int kStreamBatches = 4;
 int plan(int N, int C, int HW, Geometry* g, int* mode) {
   g->N = N;
   g->C = C;
@@ -439,8 +505,26 @@ void launch_reduce(int mode, dim3 grid, const float* x, const float* dy, const f
                    const Geometry& g) {
   hipStream_t st = tt::stream();
   if (mode == 0) bn_reduce_planes<kKind><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
+  if (mode == 3) bn_reduce_stream<kKind><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
   if (mode == 1) bn_reduce_flat<kKind, 4><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
   if (mode == 2) bn_reduce_flat<kKind, 1><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
+}
+
+// Geometry of the first sweep: the stream kernel when planes are float4-aligned, else as plan().
+int plan_reduce(int N, int C, int HW, Geometry* g, int* mode) {
+  plan(N, C, HW, g, mode);
+  if (HW % 4 != 0) return 0;
+  *mode = 3;
+  const long long vectors = (long long)N * (HW / 4);
+  const long long batch = (long long)kThreads * kStreamU;
+  long long per = kStreamBatches * batch;                 // a few batches per block ...
+  const long long min_per = (vectors + kMaxSplits - 1) / kMaxSplits;   // ... but at most kMaxSplits partials
+  if (per < min_per) per = min_per;
+  per = (per + batch - 1) / batch * batch;
+  g->per_block = (int)per;
+  g->splits = ceil_div(vectors, per);
+  g->hwv_div = tt::make_fastdiv((uint32_t)(HW / 4));
+  return 0;
 }
 
 // out[c] = sum of channel c's partials (bias gradient).
@@ -467,15 +551,16 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   const bool track = running_mean_in && running_var_in;
   TT_REQUIRE(!track || (running_mean_out && running_var_out),
              "tt_bn_fwd_train_f32: running statistics given without output buffers");
-  Geometry g;
-  int mode;
+  Geometry g, gr;
+  int mode, rmode;
   plan(N, C, HW, &g, &mode);
+  plan_reduce(N, C, HW, &gr, &rmode);
   void* ws;
-  if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
+  if (tt::workspace(sizeof(double2) * (size_t)C * gr.splits, &ws)) return -1;
   dim3 grid(g.splits, C);
   {
     tt::ProfScope prof(TT_PROF_BN_FWD_REDUCE);
-    launch_reduce<0>(mode, grid, x, x, nullptr, (double2*)ws, g);
+    launch_reduce<0>(rmode, dim3(gr.splits, C), x, x, nullptr, (double2*)ws, gr);
   }
   TT_LAUNCH_CHECK();
   FwdArgs a{};
@@ -485,6 +570,7 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   a.rm_out = running_mean_out; a.rv_out = running_var_out;
   a.given_mean = nullptr; a.given_var = nullptr;
   a.partial = (const double2*)ws;
+  a.partial_splits = gr.splits;
   a.one_minus_mom = (float)(1.0 - momentum);
   a.mom = (float)momentum;
   a.unbias = (float)((double)m / (double)(m - 1));
@@ -534,18 +620,19 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const flo
   if (check_shape("tt_bn_bwd_f32", N, C, HW)) return -1;
   TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "tt_bn_bwd_f32: null tensor pointer");
   if (!dx && !dgamma && !dbeta) return 0;
-  Geometry g;
-  int mode;
+  Geometry g, gr;
+  int mode, rmode;
   plan(N, C, HW, &g, &mode);
+  plan_reduce(N, C, HW, &gr, &rmode);
   void* ws;
-  if (tt::workspace(sizeof(double2) * (size_t)C * g.splits, &ws)) return -1;
+  if (tt::workspace(sizeof(double2) * (size_t)C * gr.splits, &ws)) return -1;
   dim3 grid(g.splits, C);
   {
     tt::ProfScope prof(TT_PROF_BN_BWD_REDUCE);
-    launch_reduce<1>(mode, grid, x, dy, save_mean, (double2*)ws, g);
+    launch_reduce<1>(rmode, dim3(gr.splits, C), x, dy, save_mean, (double2*)ws, gr);
   }
   TT_LAUNCH_CHECK();
-  BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws};
+  BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws, gr.splits};
   hipStream_t st = tt::stream();
   {
     tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
@@ -563,7 +650,7 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
   TT_REQUIRE(t && out, "tt_channel_sum_f32: null tensor pointer");
   Geometry g;
   int mode;
-  plan(N, K, HW, &g, &mode);
+  plan_reduce(N, K, HW, &g, &mode);
   void* ws;
   if (tt::workspace(sizeof(double2) * (size_t)K * g.splits, &ws)) return -1;
   launch_reduce<2>(mode, dim3(g.splits, K), t, t, nullptr, (double2*)ws, g);
