@@ -75,12 +75,31 @@ TILE_CASES = [
     (2, 40, 8, 8, 72, 1, 1, (1, 1), (0, 0), (1, 1), 1),         # plain-GEMM path, 64x64 tiles, C not a multiple of 16
     (16, 256, 14, 14, 1024, 1, 1, (1, 1), (0, 0), (1, 1), 1),   # plain-GEMM path with split left-over tiles
     (3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2),         # plain-GEMM path with groups, ragged pixel tile
+    (70, 16, 3, 3, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # tiny images: a pixel tile spans 15-29 images (buffer re-basing)
+    (5, 32, 13, 9, 48, 5, 5, (2, 1), (4, 2), (2, 1), 2),        # 25 taps, dilation + stride + groups: tap masks, negative table steps in dgrad
+    (3, 16, 14, 14, 16, 6, 6, (1, 1), (2, 2), (1, 1), 1),       # 36 taps > 31: compare-and-select addressing in all three passes
+    (2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1),       # padded 1x1: not the plain-GEMM geometry, one-tap mask
+    (4, 48, 10, 10, 24, 3, 3, (1, 1), (0, 0), (1, 1), 1),       # unpadded 3x3, rows (24) and weight rows shorter than a tile
+    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)
 ]
 
 
 @pytest.mark.parametrize('case', TILE_CASES)
 def test_conv_tile_configurations(case):
     _run_conv(case, seed=1)
+
+
+# Images too large for 32-bit byte offsets relative to a tile's (a chunk's) first image: the
+# kernels must fall back from buffer addressing to 64-bit addresses with compared bounds.
+LARGE_IMAGE_CASES = [
+XX
+    (2, 20, 3300, 3300, 4, 1, 1, (1, 1), (0, 0), (1, 1), 1),    # 871 MB per image: forward / input gradient fall back too
+]
+
+
+@pytest.mark.parametrize('case', LARGE_IMAGE_CASES)
+def test_conv_large_images_use_64_bit_addressing(case):
+    _run_conv(case, seed=3)
 
 
 def test_conv_without_bias():
