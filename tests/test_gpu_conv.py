@@ -92,7 +92,7 @@ def test_conv_tile_configurations(case):
 # Images too large for 32-bit byte offsets relative to a tile's (a chunk's) first image: the
 # kernels must fall back from buffer addressing to 64-bit addresses with compared bounds.
 LARGE_IMAGE_CASES = [
-XX
+    (2, 32, 720, 720, 8, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # 66 MB per image, a chunk may span 34 images: weight gradient falls back
     (2, 20, 3300, 3300, 4, 1, 1, (1, 1), (0, 0), (1, 1), 1),    # 871 MB per image: forward / input gradient fall back too
 ]
 
