@@ -82,6 +82,9 @@ struct Igemm {
   int voffBias;              // elements added to every lane offset so that it is never negative
   long long srdBias;         // elements subtracted from the buffer base to make up for all biases
   const void* wbuf;          // buffer modes: base of the weight operand (wp or wraw)
+  // buffer-mode input gradients of 1x1 layers read w[k][c] in place, transposed: row i of the
+  // GEMM is column c of w, so lanes (rows) are contiguous and k strides by wTransStride = C/groups
+  int wTransStride;
   // dense input-gradient launches only (all stride-parity classes as rows of one GEMM):
   // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
   const int4* rowtab;
@@ -215,7 +218,7 @@ constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out 
 
 __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
 
-template <int WM, int WN, int MT, int NT, bool SK, int MODE>
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
@@ -278,7 +281,10 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
           nmask = ~inside;   // bit 31 (the padding entries' tap) always stays set: TB*TC <= 31
         }
       }
-      if (p.wRowStride) {   // in place; rows past I are never stored
+      if constexpr (AT) {   // w[k][c] in place: k = Kred rows of I = C/groups columns per group
+        avoff = 4 * (min(i0 + arow, p.I - 1) + 4 * aq0 * p.wTransStride);
+        asoff = 4 * g * p.Kred * p.wTransStride;
+      } else if (p.wRowStride) {   // in place; rows past I are never stored
         avoff = 4 * (min(i0 + arow, p.I - 1) * p.wRowStride + 4 * aq0);
         asoff = 4 * g * p.I * p.wRowStride;
       } else {
@@ -347,7 +353,13 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
     const int q = aq0 + it * (kThreads / BM);   // always < kBKQ unless the tile has fewer than 64 rows
     if (q < kBKQ) {
       const int kq = chunk * kBKQ + q;
-      if constexpr (BUF) {
+      if constexpr (AT) {
+        // four k values of this row: one coalesced dword load each (whole chunks only)
+        const int soff = asoff + 16 * (chunk * kBKQ + it * AQ) * p.wTransStride;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          areg[it][j] = as_float(__builtin_amdgcn_raw_buffer_load_b32(wSrd, avoff, soff + 4 * j * p.wTransStride, 0));
+      } else if constexpr (BUF) {
         // in place only when rows are a whole number of chunks long: nothing to zero
         const int soff = asoff + (p.wRowStride ? 16 * (chunk * kBKQ + it * AQ) : 16 * (chunk * kBKQ + it * AQ) * p.Ipad);
         areg[it] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(wSrd, avoff, soff, 0));
@@ -721,20 +733,23 @@ TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k
 // bytes of stream-K partial accumulators for the largest tile: 2 slots per block
 size_t sk_workspace_bytes() { return (size_t)2 * kSkBlocks * 128 * 128 * sizeof(float); }
 
-template <int WM, int WN, int MT, int NT, int MODE>
+template <int WM, int WN, int MT, int NT, int MODE, bool AT>
 void launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   if (sk_blocks > 0) {
-    igemm_f32<WM, WN, MT, NT, true, MODE><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    igemm_f32<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     igemm_fixup<WM, WN, MT, NT><<<dim3(p.tiles - p.skDpTiles, MT * NT), kThreads, 0, st>>>(p);
   } else {
-    igemm_f32<WM, WN, MT, NT, false, MODE><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+    igemm_f32<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
 }
 template <int WM, int WN, int MT, int NT>
 void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
-  if (p.mode == kModeGemm) launch_mode<WM, WN, MT, NT, kModeGemm>(p, groups, sk_blocks, st);
-  else if (p.mode == kModeTapMask) launch_mode<WM, WN, MT, NT, kModeTapMask>(p, groups, sk_blocks, st);
-  else launch_mode<WM, WN, MT, NT, kModeCompare>(p, groups, sk_blocks, st);
+  const bool at = p.wTransStride > 0;
+  if (p.mode == kModeGemm && at) launch_mode<WM, WN, MT, NT, kModeGemm, true>(p, groups, sk_blocks, st);
+  else if (p.mode == kModeGemm) launch_mode<WM, WN, MT, NT, kModeGemm, false>(p, groups, sk_blocks, st);
+  else if (p.mode == kModeTapMask && at) launch_mode<WM, WN, MT, NT, kModeTapMask, true>(p, groups, sk_blocks, st);
+  else if (p.mode == kModeTapMask) launch_mode<WM, WN, MT, NT, kModeTapMask, false>(p, groups, sk_blocks, st);
+  else launch_mode<WM, WN, MT, NT, kModeCompare, false>(p, groups, sk_blocks, st);
 }
 
 // Picks how the kernel addresses the gathered operand (see Igemm::mode) and completes the table
@@ -1065,13 +1080,24 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
         p.bh = (ch + ph - r0 * dh) / sh;   // numerator is a multiple of sh by choice of r0
         p.bw = (cw + pw - s0 * dw) / sw;
         KTabArgs ka{Kred, KQ * 4, nTr, nTs, P * Q, -eh * Q, -ew, -eh, -ew, 0, 0};
+        // 1x1 layers with whole chunks of output channels: w[k][c] is read in place, transposed
+        const bool in_place = R == 1 && S == 1 && Kred % (4 * kBKQ) == 0;
         choose_mode(p, ka,
                     R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && Hx == P && Wx == Q && (P * Q) % 4 == 0,
-                    N, U, V, (long long)wp_bytes);
+                    N, U, V, in_place ? (long long)sizeof(float) * K * Cg : (long long)wp_bytes);
         tt::ProfScope prof(TT_PROF_CONV_PREP);
-        PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
-        pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
-        TT_LAUNCH_CHECK();
+        if (in_place && p.mode != kModeCompare) {
+          p.wbuf = w;
+          p.wTransStride = Cg;
+          if (p.mode == kModeTapMask) {
+            if (cached_ktab(ka, &tab)) return -1;
+            p.ktab = tab;
+          }
+        } else {
+          PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
+          pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
+          TT_LAUNCH_CHECK();
+        }
       }
       if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
     }
