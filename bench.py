@@ -42,6 +42,13 @@ RESNET50_CONVS = [
     (512, 7, 2048, 1, 1, 0, 3), (2048, 7, 512, 1, 1, 0, 2), (512, 7, 512, 3, 1, 1, 2),
 ]
 BATCH = 64
+# HBM bytes per launch of the two dominant kernels, from rocprofv3 FETCH_SIZE + WRITE_SIZE of this
+# workload (each counter scaled by what it reads for the 2 GiB copy probe of the same run: x2.0 and
+# x1.0).  Counters cannot be read from inside this script, so the figures of the last counter
+# run are carried here; the summary with the commands is in the profiles directory
+# (bench_hbm_traffic_fetch_write_size.txt).
+IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 218.6e6      # igemm_f32 + igemm_fixup, mean over the 115 launches of a step (98.6e6 algorithmic)
+BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.3e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
 
 
@@ -271,7 +278,8 @@ def main():
         'wall_ms_per_step': round(conv_wall_ms, 3),
         'roofline': {'bound': 'mfma', 'kernel': 'igemm_f32 (Conv2d forward + input gradient)',
                      'achieved': round(igemm_tflops, 2), 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': round(igemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4), 'traffic': None,
+                     'frac': round(igemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
+                     'traffic': IGEMM_TRAFFIC_BYTES_PER_LAUNCH,
                      'sustained_peak_measured': {'mean': round(mfma_mean, 1), 'min': round(mfma_min, 1),
                                                  'max': round(mfma_max, 1), 'unit': 'TFLOP/s',
                                                  'what': '100 launches of dense v_mfma_f32_32x32x2_f32, '
@@ -289,7 +297,8 @@ def main():
                'per_shape_gbs': per_shape,
                'roofline': {'bound': 'hbm', 'kernel': 'bn_bwd_apply (reads x, dy; writes dx)',
                             'achieved': round(bwd_apply_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                            'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4), 'traffic': None,
+                            'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4),
+                            'traffic': BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH,
                             'sustained_measured': {'read_gbs': round(hbm_read, 1), 'copy_gbs': round(hbm_copy, 1),
                                                    'what': '2 GiB streamed, 16 KiB contiguous per block'},
                             'avg_launch_ms': round(ms_ba / max(1, n_ba), 5)},
