@@ -218,6 +218,16 @@ constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out 
 
 __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
 
+// s_waitcnt vmcnt(0) in straight-line code.  Stores share the counter with loads, and the
+// compiler, unsure after a branch whether an earlier load has been waited for, repeats the wait
+// in every conditional store block -- which then waits for the stores before it.  One explicit
+// wait before the first store lets it drop those.
+__device__ __forceinline__ void wait_loads() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0), expcnt and lgkmcnt left alone
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
   static_assert(WM * WN == 4, "four waves per block");
@@ -532,18 +542,29 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       obase[y] = (uint32_t)((int)n * p.outStrideN + g * p.outStrideG + ((int)u * p.ou + p.ouh) * p.outRow +
                             (int)v * p.ov + p.ovw);
     }
+    // Everything the stores need is fetched before the first store: a wait for a load issued
+    // between stores would also wait for every store before it (one counter covers both), and
+    // the epilogue would run at one store round trip per row.
     if (p.rowtab == nullptr) {
+      float bz[MT][16];
+#pragma unroll
+      for (int x = 0; x < MT; ++x)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+          bz[x][r] = p.bias ? p.bias[g * p.I + min(i, p.I - 1)] : 0.f;
+        }
+      wait_loads();
 #pragma unroll
       for (int x = 0; x < MT; ++x) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
           if (i < p.I) {
-            const float bz = p.bias ? p.bias[g * p.I + i] : 0.f;
             const uint32_t ioff = (uint32_t)(i * p.outStrideI);
 #pragma unroll
             for (int y = 0; y < NT; ++y)
-              if (mok[y]) p.out[obase[y] + ioff] = acc[x][y][r] + bz;
+              if (mok[y]) p.out[obase[y] + ioff] = acc[x][y][r] + bz[x][r];
           }
         }
       }
@@ -560,19 +581,33 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
         oh[y] = (int)u * p.ou;
         ow[y] = (int)(rem - u * p.divV.d) * p.ov;
       }
+      // eight rows at a time: their table entries and biases are loaded, then stored to
 #pragma unroll
       for (int x = 0; x < MT; ++x) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-          if (i < p.I) {
-            const int4 e = p.rowtab[i];
-            const float bz = p.bias ? p.bias[e.w] : 0.f;
+        for (int r0 = 0; r0 < 16; r0 += 8) {
+          int4 row[8];
+          float bz[8];
 #pragma unroll
-            for (int y = 0; y < NT; ++y)
-              if (mok[y] && oh[y] + e.y < p.outH && ow[y] + e.z < p.outW)
-                p.out[obase[y] + (uint32_t)e.x] = acc[x][y][r] + bz;
+          for (int r = 0; r < 8; ++r) {
+            const int i = i0 + (wm * MT + x) * 32 + 8 * ((r0 + r) >> 2) + 4 * h + (r & 3);
+            row[r] = p.rowtab[min(i, p.I - 1)];
           }
+#pragma unroll
+          for (int r = 0; r < 8; ++r) bz[r] = p.bias ? p.bias[row[r].w] : 0.f;
+          wait_loads();
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            const int i = i0 + (wm * MT + x) * 32 + 8 * ((r0 + r) >> 2) + 4 * h + (r & 3);
+            if (i < p.I) {
+              const int4 e = row[r];
+#pragma unroll
+              for (int y = 0; y < NT; ++y)
+                if (mok[y] && oh[y] + e.y < p.outH && ow[y] + e.z < p.outW)
+                  p.out[obase[y] + (uint32_t)e.x] = acc[x][y][r0 + r] + bz[r];
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -675,10 +710,17 @@ __global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p) {
   const uint32_t u = tt::fd_div(rem, p.divV);
   const uint32_t v = rem - u * p.divV.d;
   const uint32_t obase = (uint32_t)((int)n * p.outStrideN + ((int)u * p.ou + p.ouh) * p.outRow + (int)v * p.ov + p.ovw);
+  float bz[16];   // all loads before the first store (see the epilogue of igemm_f32)
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-    if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[r >> 2][r & 3] + (p.bias ? p.bias[i] : 0.f);
+    bz[r] = p.bias ? p.bias[min(i, p.I - 1)] : 0.f;
+  }
+  wait_loads();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+    if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[r >> 2][r & 3] + bz[r];
   }
 }
 
