@@ -20,6 +20,8 @@
 // masked when the values are written to LDS.  Offsets are relative to the first image of the
 // chunk; geometries whose offsets could reach 2 GiB, or with more than 31 taps, take the
 // compare-and-select path instead.
+#include <map>
+
 #include "tt_common.h"
 
 namespace {
@@ -50,6 +52,9 @@ struct Wgrad {
   int xBias;                  // buffer path: ph*W + pw, keeps lane offsets non-negative
   tt::FastDiv divDh, divDw;   // buffer path: division by the dilation
   uint32_t rowOnes;           // buffer path: bit r*S set for every tap row r
+  // buffer path: per output pixel m {image n, 4*(p*Q + q), 4*(ih*W + iw + xBias), tap mask};
+  // entries from M to chunks*32 hold {N-1, bit 31, 0, all ones}.  Built once per geometry.
+  const int4* pixtab;
 };
 
 constexpr int kSrdFlags = 0x00020000;     // raw buffer, 32-bit data format
@@ -67,13 +72,38 @@ __device__ __forceinline__ uint32_t tap_range_bits(int pos, int lim, int n, int 
   return lo > hi ? 0u : upto & ~below;
 }
 
+// Pixel table of the buffer path: what the main loop would otherwise recompute for every chunk
+// in every block (two divisions, the tap ranges) depends only on the geometry.
+__global__ void wgrad_build_pixtab(int4* __restrict__ tab, Wgrad p, int entries, int N) {
+  const int m = blockIdx.x * blockDim.x + threadIdx.x;
+  if (m >= entries) return;
+  int4 e = make_int4(N - 1, (int)0x80000000u, 0, -1);
+  if (m < p.M) {
+    const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
+    const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
+    const uint32_t pp = tt::fd_div(pq, p.divQ);
+    const uint32_t qq = pq - pp * p.divQ.d;
+    const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
+    // valid tap columns, replicated into every valid tap row (fields of S bits: no carries)
+    const uint32_t cols = tap_range_bits(iw, p.W, p.S, 1, p.divDw);
+    const uint32_t rows = tap_range_bits(ih, p.H, p.R, p.S, p.divDh) & p.rowOnes;
+    e = make_int4((int)n, 4 * (int)pq, 4 * (ih * p.W + iw + p.xBias), (int)~(cols * rows));   // bit 31 stays set: R*S <= 31
+  }
+  tab[m] = e;
+}
+
 // Two blocks per CU is all the LDS tiles allow: tell the compiler not to squeeze registers (and
 // spill) for a third wave per SIMD.
-template <int WM, int WN, int MT, int NT, bool BUF>
+// VA / VB (buffer path only): dy / x are fetched as 16-byte vectors of four consecutive pixels
+// (thread = (row group of 32, pixel quad) instead of (row group of 8, pixel)).  VA needs P*Q to be
+// a multiple of 4 so that a quad never straddles two images, VB in addition a 1x1, stride-1,
+// unpadded layer, where x is indexed by the output pixel like dy and has no padding to mask.
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_f32(const Wgrad p) {
   static_assert(WM * WN == 4, "four waves per block");
+  static_assert(BUF || (!VA && !VB), "vector fetches belong to the buffer path");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
-  constexpr int A_ROWS = BM / 8, B_ROWS = BN / 8;   // rows per thread (8 row groups of 32 lanes)
+  constexpr int A_ROWS = VA ? BM / 32 : BM / 8, B_ROWS = VB ? BN / 32 : BN / 8;   // fetches per thread and chunk
   __shared__ __attribute__((aligned(16))) float As[2][BM][kLd];
   __shared__ __attribute__((aligned(16))) float Bs[2][BN][kLd];
   // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}; buffer path: {4 * offset, tap r*S + s}
@@ -105,6 +135,7 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   }
 
   const int px = tid & 31, rg = tid >> 5;   // this thread's pixel inside a chunk, and row group
+  const int qpx = tid & 7, rgq = tid >> 3;   // vector fetches: pixel quad inside a chunk, and row group
   const float* __restrict__ dyg = p.dy + (size_t)g * p.dyStrideG;
   const float* __restrict__ xg = p.x + (size_t)g * p.xStrideG;
 
@@ -128,34 +159,43 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   int aoff[A_ROWS];
   if constexpr (BUF) {
 #pragma unroll
-    for (int t = 0; t < A_ROWS; ++t) aoff[t] = 4 * min(arow + 8 * t, p.Kg - 1) * p.PQ;   // rows past Kg are never stored
+    for (int t = 0; t < A_ROWS; ++t)   // rows past Kg are never stored
+      aoff[t] = 4 * min(VA ? i0 + rgq + 32 * t : arow + 8 * t, p.Kg - 1) * p.PQ;
+  }
+  // vector fetches: offsets of the quad's first pixel, staging vectors, per-row x offsets
+  uint32_t qvoff = 0x80000000u, qxvoff = 0x80000000u;
+  floatx4 aregv[VA ? A_ROWS : 1], bregv[VB ? B_ROWS : 1];
+  int boffv[VB ? B_ROWS : 1];
+  if constexpr (VB) {
+#pragma unroll
+    for (int t = 0; t < B_ROWS; ++t) boffv[t] = 4 * min(j0 + rgq + 32 * t, p.J - 1) * p.HW;   // column j = channel
   }
 
-  auto decompose = [&](int chunk) __attribute__((always_inline)) {
+  // table entry of this lane's pixel in the chunk after the one being decomposed: fetched one
+  // chunk ahead so that its latency is covered
+  int4 pixnext = make_int4(0, 0, 0, 0);
+  int2 pixnextq = make_int2(0, 0);
+  auto fetch_pix = [&](int chunk) __attribute__((always_inline)) {
+    if constexpr (BUF && !(VA && VB)) pixnext = p.pixtab[chunk * kBK + px];
+    if constexpr (VA || VB) pixnextq = *reinterpret_cast<const int2*>(&p.pixtab[chunk * kBK + 4 * qpx]);
+  };
+  auto decompose = [&](int chunk, int following) __attribute__((always_inline)) {
     if constexpr (BUF) {
-      const int mfirst = __builtin_amdgcn_readfirstlane(chunk * kBK);
-      const uint32_t n0 = tt::fd_div((uint32_t)mfirst, p.divPQ);
+      const int4 e = pixnext;   // entry of `chunk`
+      const int2 eq = pixnextq;
+      fetch_pix(following);
+      const int n0 = __builtin_amdgcn_readfirstlane((VA && VB) ? eq.x : e.x);   // lane 0 holds the chunk's first pixel
+      if constexpr (VA || VB) {
+        qvoff = (uint32_t)(4 * (eq.x - n0) * p.dyStrideN) + (uint32_t)eq.y;   // bit 31 of eq.y: quad past the end
+        qxvoff = (uint32_t)(4 * (eq.x - n0) * p.xStrideN) + (uint32_t)eq.y;   // 1x1: x is indexed like dy
+      }
       dySrd = __builtin_amdgcn_make_buffer_rsrc((void*)(p.dy + ((size_t)n0 * p.dyStrideN + (size_t)g * p.dyStrideG)), 0,
                                                 kSrdRecords, kSrdFlags);
       xSrd = __builtin_amdgcn_make_buffer_rsrc(
           (void*)(p.x + ((long long)n0 * p.xStrideN + (long long)g * p.xStrideG - p.xBias)), 0, kSrdRecords, kSrdFlags);
-      const int m = chunk * kBK + px;
-      dyvoff = 0x80000000u;
-      xvoff = 0;
-      nmask = 0xffffffffu;
-      if (m < p.M) {
-        const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
-        const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
-        const uint32_t pp = tt::fd_div(pq, p.divQ);
-        const uint32_t qq = pq - pp * p.divQ.d;
-        const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
-        dyvoff = 4u * (uint32_t)((int)(n - n0) * p.dyStrideN + (int)pq);
-        xvoff = 4u * (uint32_t)((int)(n - n0) * p.xStrideN + ih * p.W + iw + p.xBias);
-        // valid tap columns, replicated into every valid tap row (fields of S bits: no carries)
-        const uint32_t cols = tap_range_bits(iw, p.W, p.S, 1, p.divDw);
-        const uint32_t rows = tap_range_bits(ih, p.H, p.R, p.S, p.divDh) & p.rowOnes;
-        nmask = ~(cols * rows);   // bit 31 (columns past J) stays set: R*S <= 31
-      }
+      dyvoff = (uint32_t)(4 * (e.x - n0) * p.dyStrideN) + (uint32_t)e.y;   // bit 31 of e.y survives: pixel past the end
+      xvoff = (uint32_t)(4 * (e.x - n0) * p.xStrideN) + (uint32_t)e.z;
+      nmask = (uint32_t)e.w;
       return;
     }
     const int m = chunk * kBK + px;
@@ -176,12 +216,19 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   auto load_step = [&](int li) __attribute__((always_inline)) {
     if constexpr (BUF) {
       if (li < A_ROWS) {
-        areg[li] = as_float(__builtin_amdgcn_raw_buffer_load_b32(dySrd, (int)(dyvoff + (uint32_t)aoff[li]), 0, 0));
+        if constexpr (VA)
+          aregv[li] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(dySrd, (int)(qvoff + (uint32_t)aoff[li]), 0, 0));
+        else
+          areg[li] = as_float(__builtin_amdgcn_raw_buffer_load_b32(dySrd, (int)(dyvoff + (uint32_t)aoff[li]), 0, 0));
       } else {
         const int t = li - A_ROWS;
-        const int2 e = jreg[t];
-        const uint32_t vo = ((nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
-        breg[t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
+        if constexpr (VB) {
+          bregv[t] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(xSrd, (int)(qxvoff + (uint32_t)boffv[t]), 0, 0));
+        } else {
+          const int2 e = jreg[t];
+          const uint32_t vo = ((nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
+          breg[t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
+        }
       }
       return;
     }
@@ -203,8 +250,14 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   // outside the image must be exactly zero: AND with an all-ones / all-zeros word.
   auto store_step = [&](int buf, int li) __attribute__((always_inline)) {
     if constexpr (BUF) {   // padding and pixels past the end were read as zeros
-      if (li < A_ROWS) As[buf][rg + 8 * li][px] = areg[li];
-      else Bs[buf][rg + 8 * (li - A_ROWS)][px] = breg[li - A_ROWS];
+      if (li < A_ROWS) {
+        if constexpr (VA) *reinterpret_cast<floatx4*>(&As[buf][rgq + 32 * li][4 * qpx]) = aregv[li];
+        else As[buf][rg + 8 * li][px] = areg[li];
+      } else {
+        const int t = li - A_ROWS;
+        if constexpr (VB) *reinterpret_cast<floatx4*>(&Bs[buf][rgq + 32 * t][4 * qpx]) = bregv[t];
+        else Bs[buf][rg + 8 * t][px] = breg[t];
+      }
       return;
     }
     if (li < A_ROWS) {
@@ -247,7 +300,7 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   constexpr int LPS = (L + T / 2 - 2) / (T / 2 - 1);       // loads per slot, slots 1 .. T/2-1
   constexpr int kStore = 5 * T / 8, kSync = T - 4;
   constexpr int SPS = (L + (kSync - kStore) - 1) / (kSync - kStore);   // LDS writes per slot
-  auto chunk_body = [&](const int buf, const int nchunk) __attribute__((always_inline)) {
+  auto chunk_body = [&](const int buf, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < T; ++s) {
       const int kk = s / PK, rem = s % PK;
@@ -255,7 +308,7 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
       acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x2f32(opA[kk & 1][xx][j], opB[kk & 1][yy][j], acc[xx][yy], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
       if (rem == 0 && kk < 3) read_ops((kk + 1) & 1, buf, kk + 1);
-      if (s == 0) decompose(nchunk);
+      if (s == 0) decompose(nchunk, nnchunk);
 #pragma unroll
       for (int u = 0; u < LPS; ++u) {
         const int li = (s - 1) * LPS + u;
@@ -275,12 +328,15 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   };
 
   __syncthreads();   // jtab
+  if constexpr (!VB) {
 #pragma unroll
-  for (int t = 0; t < B_ROWS; ++t) jreg[t] = jtab[rg + 8 * t];
+    for (int t = 0; t < B_ROWS; ++t) jreg[t] = jtab[rg + 8 * t];
+  }
 
   if (c_begin < c_end) {
     const int last = c_end - 1;
-    decompose(c_begin);
+    fetch_pix(c_begin);
+    decompose(c_begin, min(c_begin + 1, last));
 #pragma unroll
     for (int li = 0; li < L; ++li) load_step(li);
 #pragma unroll
@@ -290,10 +346,10 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
     // past the end the last chunk is fetched again (cache hits) instead of branching
     int c = c_begin;
     for (; c + 1 < c_end; c += 2) {
-      chunk_body(0, c + 1);
-      chunk_body(1, min(c + 2, last));
+      chunk_body(0, c + 1, min(c + 2, last));
+      chunk_body(1, min(c + 2, last), min(c + 3, last));
     }
-    if (c < c_end) chunk_body(0, last);
+    if (c < c_end) chunk_body(0, last, last);
   }
 
   float* __restrict__ out = p.out + (size_t)split * p.outStrideSplit + (size_t)g * p.Kg * p.J;
@@ -358,10 +414,45 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce(const float* __restrict
 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+struct PixKey {
+  int v[14];
+  bool operator<(const PixKey& o) const {
+    for (int i = 0; i < 14; ++i)
+      if (v[i] != o.v[i]) return v[i] < o.v[i];
+    return false;
+  }
+};
+// The pixel table depends only on the geometry: built on first use, kept for the process
+// (16 bytes per output pixel; at most kMaxPixTables geometries, then the oldest are dropped).
+constexpr size_t kMaxPixTables = 256;
+int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
+  static std::map<PixKey, int4*> cache;
+  const PixKey key{{N, P, Q, p.H, p.W, p.sh, p.sw, p.ph, p.pw, p.dh, p.dw, p.R, p.S, p.chunks}};
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    hipStream_t st = tt::stream();
+    if (cache.size() >= kMaxPixTables) {
+      TT_HIP(hipStreamSynchronize(st));
+      for (auto& kv : cache) TT_HIP(hipFree(kv.second));
+      cache.clear();
+    }
+    const int entries = p.chunks * kBK;
+    int4* tab = nullptr;
+    TT_HIP(hipMalloc((void**)&tab, sizeof(int4) * (size_t)entries));
+    wgrad_build_pixtab<<<ceil_div(entries, 256), 256, 0, st>>>(tab, p, entries, N);
+    TT_LAUNCH_CHECK();
+    it = cache.emplace(key, tab).first;
+  }
+  *out = it->second;
+  return 0;
+}
+
 template <int WM, int WN, int MT, int NT>
-void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, hipStream_t st) {
-  if (buf) wgrad_f32<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
-  else wgrad_f32<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
+void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStream_t st) {
+  if (buf && va && vb) wgrad_f32<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
+  else if (buf && va) wgrad_f32<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
+  else if (buf) wgrad_f32<WM, WN, MT, NT, true, false, false><<<grid, kThreads, 0, st>>>(p);
+  else wgrad_f32<WM, WN, MT, NT, false, false, false><<<grid, kThreads, 0, st>>>(p);
 }
 
 }  // namespace
@@ -437,18 +528,22 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
                                ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
   const bool buf = R * S <= 31 && reach < (1LL << 31) - (1LL << 20);
+  if (buf && cached_pixtab(p, N, P, Q, &p.pixtab)) return -1;
+  // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
+  const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)dy & 15) == 0;
+  const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)x & 15) == 0;
   dim3 grid(tilesI * tilesJ, groups, splits);
   hipStream_t st = tt::stream();
   {
     tt::ProfScope prof(TT_PROF_CONV_WGRAD);
     if (bm == 128 && bn == 128)
-      launch_wgrad<2, 2, 2, 2>(p, grid, buf, st);
+      launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, st);
     else if (bm == 64 && bn == 128)
-      launch_wgrad<2, 2, 1, 2>(p, grid, buf, st);
+      launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, st);
     else if (bm == 128 && bn == 64)
-      launch_wgrad<2, 2, 2, 1>(p, grid, buf, st);
+      launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, st);
     else
-      launch_wgrad<2, 2, 1, 1>(p, grid, buf, st);
+      launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, st);
   }
   TT_LAUNCH_CHECK();
   if (splits > 1) {
