@@ -228,8 +228,10 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// The kernel body: `block_x` is the block's index among the blocks of launch `p` (a launch may
+// be one of several that share a grid, see igemm_multi_f32).
 template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
-__global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
+__device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
@@ -615,7 +617,7 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
 
   const int chunks = p.KQ / kBKQ;
   if constexpr (!SK) {
-    set_tile(xcd_remap(blockIdx.x, p.tiles));
+    set_tile(xcd_remap(block_x, p.tiles));
     run_segment(0, chunks);
     epilogue();
   } else {
@@ -671,6 +673,27 @@ __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
       __syncthreads();   // the next segment's first stores reuse LDS buffer 0
     }
   }
+}
+
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
+__global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT>(p, (int)blockIdx.x);
+}
+
+// Several data-parallel launches in one grid (the stride-parity classes of a strided input
+// gradient): blocks [first[i], first[i+1]) belong to launch i.  One grid instead of a short
+// launch per class, each with its own ramp-up and tail.
+constexpr int kMaxMulti = 4;
+struct IgemmMulti {
+  Igemm c[kMaxMulti];
+  int first[kMaxMulti + 1];
+  int n;
+};
+template <int WM, int WN, int MT, int NT, int MODE>
+__global__ __launch_bounds__(kThreads, 2) void igemm_multi_f32(const IgemmMulti m) {
+  int ci = 0;
+  while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
+  igemm_body<WM, WN, MT, NT, false, MODE, false>(m.c[ci], (int)blockIdx.x - m.first[ci]);
 }
 
 // Stream-K second stage: MT*NT blocks per left-over tile, one per 32x32 accumulator tile of
@@ -850,6 +873,36 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
     launch_config<1, 4, 1, 2>(p, groups, t.sk_blocks, st);
   else
     launch_config<2, 2, 1, 1>(p, groups, t.sk_blocks, st);
+  TT_LAUNCH_CHECK();
+  return 0;
+}
+
+// Launches the data-parallel GEMMs in `list` (same tile shape, same addressing mode, no stream-K,
+// no transposed weights) as one grid.
+template <int WM, int WN, int MT, int NT>
+void launch_multi_config(const IgemmMulti& m, int groups, hipStream_t st) {
+  const dim3 grid(m.first[m.n], groups);
+  if (m.c[0].mode == kModeTapMask) igemm_multi_f32<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
+  else igemm_multi_f32<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
+}
+int launch_igemm_multi(IgemmMulti& m, int groups, TileChoice t, int prof_id) {
+  tt::ProfScope prof(prof_id);
+  m.first[0] = 0;
+  for (int i = 0; i < m.n; ++i) {
+    Igemm& p = m.c[i];
+    p.tilesI = p.Ipad / t.bm;
+    p.tiles = p.tilesI * ceil_div(p.M, t.bn);
+    m.first[i + 1] = m.first[i] + p.tiles;
+  }
+  hipStream_t st = tt::stream();
+  if (t.bm == 128 && t.bn == 128)
+    launch_multi_config<2, 2, 2, 2>(m, groups, st);
+  else if (t.bm == 64 && t.bn == 256)
+    launch_multi_config<1, 4, 2, 2>(m, groups, st);
+  else if (t.bm == 32 && t.bn == 256)
+    launch_multi_config<1, 4, 1, 2>(m, groups, st);
+  else
+    launch_multi_config<2, 2, 1, 1>(m, groups, st);
   TT_LAUNCH_CHECK();
   return 0;
 }
@@ -1083,6 +1136,12 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       if (((cw + pw - s2 * dw) % sw + sw) % sw == 0) { ++tap_cols; break; }
   const bool allow_stream_k = tap_rows * tap_cols <= 1;
 
+  // Classes that have taps and agree on tile shape and addressing mode go into one grid when
+  // there are 2..kMaxMulti of them; anything else is launched on its own.
+  IgemmMulti multi{};
+  TileChoice multi_tile{};
+  bool multi_ok = !allow_stream_k && tap_rows * tap_cols <= kMaxMulti;
+
   int slot = 0;
   for (int ch = 0; ch < sh && ch < Hx; ++ch) {
     // taps r with (ch + ph - r*dh) % sh == 0
@@ -1141,8 +1200,26 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
           TT_LAUNCH_CHECK();
         }
       }
+      if (multi_ok && KQ > 0 && t.sk_blocks == 0 && p.wTransStride == 0 && p.mode != kModeGemm &&
+          (multi.n == 0 || (t.bm == multi_tile.bm && t.bn == multi_tile.bn && p.mode == multi.c[0].mode))) {
+        // longest reduction first: the heavy blocks start early, the light ones fill the tail
+        int at = multi.n;
+        while (at > 0 && multi.c[at - 1].KQ < p.KQ) {
+          multi.c[at] = multi.c[at - 1];
+          --at;
+        }
+        multi.c[at] = p;
+        ++multi.n;
+        multi_tile = t;
+        continue;
+      }
       if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
     }
+  }
+  if (multi.n == 1) {
+    if (launch_igemm(multi.c[0], groups, multi_tile, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
+  } else if (multi.n > 1) {
+    if (launch_igemm_multi(multi, groups, multi_tile, TT_PROF_CONV_IGEMM_DGRAD)) return -1;
   }
   return 0;
 }
