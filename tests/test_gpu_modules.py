@@ -128,6 +128,101 @@ def test_preact_block_on_device_matches_oracle_composition():
     _close(bn2.bias.grad.get(), db2_ref, atol=2e-5, name='dbeta2')
 
 
+def test_dcgan_generator_stack_matches_oracle_composition():
+    """ConvTranspose2d 100->512 (k4 s1 p0), then k4 s2 p1: 512->256->128->64->3, BatchNorm2d + ReLU
+    in between, no bias: the baseline's conv-transpose configuration at batch 8, through
+    nn.Sequential on the device, against the same stack composed from oracle calls."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    tt.manual_seed(0)
+    chans = [100, 512, 256, 128, 64, 3]
+    geo = [((1, 1), (0, 0))] + [((2, 2), (1, 1))] * 4
+    layers = []
+    for i in range(5):
+        layers.append(nn.ConvTranspose2d(chans[i], chans[i + 1], 4, stride=geo[i][0], padding=geo[i][1], bias=False))
+        if i < 4:
+            layers += [nn.BatchNorm2d(chans[i + 1]), nn.ReLU()]
+    net = nn.Sequential(*layers)
+    ws = [np.asarray(m.weight.data).copy() for m in layers if isinstance(m, nn.ConvTranspose2d)]
+
+    def relu_margin(z):
+        """Smallest |pre-activation| any ReLU of the stack sees (float32 oracle forward)."""
+        a, margin = z, np.inf
+        for i in range(4):
+            a = oracle.transposed_convolution_forward(a, ws[i], None, geo[i][0], geo[i][1], (0, 0), (1, 1), 1)
+            c = chans[i + 1]
+            a, _, _, _ = oracle.batch_norm_forward(a, np.ones(c, np.float32), np.zeros(c, np.float32), None, None,
+                                                   True, 0.1, 1e-5)
+            margin = min(margin, float(np.abs(a).min()))
+            a = np.maximum(a, 0)
+        return margin
+
+    # ReLU is discontinuous in its gradient: a pre-activation within rounding distance of zero may
+    # get a different mask from two correct float32 evaluations, and the gradients then differ by
+    # a whole element.  Draw inputs until every pre-activation keeps a safe distance from zero.
+    for _ in range(50):
+        z = np.random.randn(8, 100, 1, 1).astype(np.float32)
+        if relu_margin(z) > 1e-6:   # device and oracle pre-activations differ by ~1e-7
+            break
+    else:
+        pytest.fail('no input with a safe ReLU margin found')
+    g = np.random.randn(8, 3, 64, 64).astype(np.float32)
+
+    def oracle_stack(dtype):
+        """Forward and backward of the stack composed from oracle calls in `dtype`."""
+        a, tape = z.astype(dtype), []
+        wd = [w.astype(dtype) for w in ws]
+        for i in range(5):
+            st, pd = geo[i]
+            y = oracle.transposed_convolution_forward(a, wd[i], None, st, pd, (0, 0), (1, 1), 1)
+            tape.append(('convt', a, i))
+            a = y
+            if i < 4:
+                c = chans[i + 1]
+                y, saved, _, _ = oracle.batch_norm_forward(a, np.ones(c, dtype), np.zeros(c, dtype), None, None,
+                                                           True, 0.1, 1e-5)
+                tape.append(('bn', a, saved, c))
+                a = np.maximum(y, 0)
+                tape.append(('relu', a))
+        grad, dws, dgs = g.astype(dtype), {}, {}
+        for rec in reversed(tape):
+            if rec[0] == 'relu':
+                grad = grad * (rec[1] > 0)
+            elif rec[0] == 'bn':
+                grad, dgs[rec[3]], _ = oracle.batch_norm_backward(grad, rec[1], np.ones(rec[3], dtype), rec[2])
+            else:
+                st, pd = geo[rec[2]]
+                grad, dws[rec[2]], _ = oracle.transposed_convolution_backward(grad, rec[1], wd[rec[2]], st, pd, (1, 1), 1)
+        return a, grad, dws, dgs
+
+    out_ref, dz_ref, dws, dgs = oracle_stack(np.float32)
+    out64, dz64, dws64, dgs64 = oracle_stack(np.float64)
+
+    def check(got, ref32, ref64, name):
+        # Rounding differences compound through five layers and four BatchNorm backward passes
+        # (cancellation), so two correct float32 evaluations differ by more than one layer's
+        # tolerance: the device result must be as close to the float64 stack as the oracle's.
+        scale = float(np.abs(ref64).max())
+        err_gpu = float(np.abs(got - ref64).max()) / scale
+        err_cpu = float(np.abs(ref32 - ref64).max()) / scale
+        assert err_gpu <= max(3 * err_cpu, 2e-5), f'{name}: device err {err_gpu:.3g} vs oracle err {err_cpu:.3g}'
+
+    net.cuda()
+    zt = tt.tensor(z, requires_grad=True)
+    out = net(zt.cuda())
+    assert out.shape == (8, 3, 64, 64)
+    out.backward(tt.tensor(g).cuda())
+    _close(out.cpu().detach().numpy(), out_ref, atol=2e-5, name='out')
+    check(out.cpu().detach().numpy(), out_ref, out64, 'out')
+    check(zt.grad, dz_ref, dz64, 'dz')
+    convs = [m for m in layers if isinstance(m, nn.ConvTranspose2d)]
+    for i, m in enumerate(convs):
+        check(m.weight.grad.get(), dws[i], dws64[i], f'dw{i}')
+    bns = [m for m in layers if isinstance(m, nn.BatchNorm2d)]
+    for m in bns:
+        check(m.weight.grad.get(), dgs[m.num_features], dgs64[m.num_features], f'dgamma{m.num_features}')
+
+
 def test_unbatched_input_and_mixed_device_error():
     import pytortto_amd as tt
     tt.manual_seed(5)
