@@ -65,7 +65,9 @@ enum {
   TT_PROF_BN_FWD_APPLY = 6,
   TT_PROF_BN_BWD_REDUCE = 7,
   TT_PROF_BN_BWD_APPLY = 8,
-  TT_PROF_COUNT = 9
+  TT_PROF_MAXPOOL_FWD = 9,
+  TT_PROF_MAXPOOL_BWD = 10,
+  TT_PROF_COUNT = 11
 };
 int tt_profile_enable(int on);
 int tt_profile_read(int kernel_id, long long* launches, double* total_ms);
@@ -141,11 +143,33 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
                   const float* save_mean, const float* save_var_eps, const float* save_sd,
                   float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
 
+/* ---- MaxPool2d (autograd/grad_nn.py:784-864) ------------------------------------------------ */
+
+/* x: [NC, H, W] planes (N*C of them), y and tap: [NC, P, Q].  Windows are taken over x padded
+ * with -inf (padding ph/pw; taps beyond the bottom/right edge, as ceil_mode produces, read -inf
+ * too); NaN is ignored, the first maximum in (kernel row, kernel column) order wins and `tap`
+ * receives kernel_row * kw + kernel_column (_max_pool2d, :784-808; the reference's `pos` tuple
+ * holds the same two indices).  P and Q are chosen by the caller (floor or ceil rule, :566-579);
+ * every window must start inside the input or its top/left padding. */
+int tt_maxpool2d_fwd_f32(const float* x, float* y, int* tap, int NC, int H, int W, int P, int Q,
+                         int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw);
+/* dx[NC, H, W] from dy[NC, P, Q] and the forward's `tap` (_max_pool2d_backward, :811-824): each
+ * output gradient is ASSIGNED to its window's arg-max pixel; when overlapping windows chose the
+ * same pixel the last window in (p, q) order wins, as NumPy's indexed assignment does -- the
+ * reference does not sum them.  Pixels no window chose receive 0. */
+int tt_maxpool2d_bwd_f32(const float* dy, const int* tap, float* dx, int NC, int H, int W, int P, int Q,
+                         int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw);
+
 /* ---- elementwise glue so whole stacks stay on the device ----------------------------------- */
 
 /* y = max(x, 0) (autograd/grad_nn.py:33-69); dx = dy * (y > 0). */
 int tt_relu_fwd_f32(const float* x, float* y, size_t n);
 int tt_relu_bwd_f32(const float* dy, const float* y, float* dx, size_t n);
+/* y = maximum(x * negative_slope, x); dx = dy where x >= 0 (or NaN), dy * negative_slope where
+ * x < 0 (autograd/grad_nn.py:71-95).  dx may alias dy: the reference scales the incoming
+ * gradient array in place (:94). */
+int tt_leaky_relu_fwd_f32(const float* x, float* y, float negative_slope, size_t n);
+int tt_leaky_relu_bwd_f32(const float* dy, const float* x, float* dx, float negative_slope, size_t n);
 /* out = a + b (residual Add, autograd/grad_fcn.py:177-203). */
 int tt_add_f32(const float* a, const float* b, float* out, size_t n);
 /* acc += alpha * v: gradient accumulation `fn.grad[ind] += grad` (tensor.py:596-599,

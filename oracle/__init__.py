@@ -19,6 +19,11 @@ publishes no golden vectors for this path):
                         running-stat recurrence, sum(dx)=0, sum(dx*xhat)=0,
                         torch CPU ``F.batch_norm`` + autograd, float64 finite differences
 
+* ``max_pool2d*``       nested-loop brute force with sequential assignment (last window wins),
+                        torch CPU ``F.max_pool2d`` (forward always; backward where windows do
+                        not overlap, so that assignment and summation coincide)
+* ``relu*/leaky_relu*`` closed forms on signs / zero / NaN, torch CPU with autograd
+
 The checks live in ``tests/test_oracle_*.py``.
 """
 from .conv import (conv2d, conv2d_backward_w, conv2d_backward_x, conv_output_size,
@@ -26,10 +31,14 @@ from .conv import (conv2d, conv2d_backward_w, conv2d_backward_x, conv_output_siz
                    transposed_convolution_forward, transposed_convolution_backward)
 from .batchnorm import batch_norm_forward, batch_norm_backward
 from .nninit import conv_parameters, bn_affine_c4
+from .pool import max_pool2d, max_pool2d_backward, pool_output_size
+from .activation import relu_forward, relu_backward, leaky_relu_forward, leaky_relu_backward
 
 __all__ = [
     'conv2d', 'conv2d_backward_w', 'conv2d_backward_x', 'conv_output_size',
     'conv_transpose_output_size', 'convolution_forward', 'convolution_backward',
     'transposed_convolution_forward', 'transposed_convolution_backward',
     'batch_norm_forward', 'batch_norm_backward', 'conv_parameters', 'bn_affine_c4',
+    'max_pool2d', 'max_pool2d_backward', 'pool_output_size',
+    'relu_forward', 'relu_backward', 'leaky_relu_forward', 'leaky_relu_backward',
 ]

@@ -43,6 +43,10 @@ PROTOTYPES = {
     'tt_bn_bwd_f32': [_P] * 9 + [_I, _I, _I],
     'tt_relu_fwd_f32': [_P, _P, c_size_t],
     'tt_relu_bwd_f32': [_P, _P, _P, c_size_t],
+    'tt_leaky_relu_fwd_f32': [_P, _P, c_float, c_size_t],
+    'tt_leaky_relu_bwd_f32': [_P, _P, _P, c_float, c_size_t],
+    'tt_maxpool2d_fwd_f32': [_P, _P, _P] + [_I] * 13,
+    'tt_maxpool2d_bwd_f32': [_P, _P, _P] + [_I] * 13,
     'tt_add_f32': [_P, _P, _P, c_size_t],
     'tt_axpy_f32': [c_float, _P, _P, c_size_t],
     'tt_fill_f32': [_P, c_float, c_size_t],
@@ -110,7 +114,7 @@ def device_info():
 
 PROF_KERNELS = {
     'conv_igemm_fwd': 0, 'conv_igemm_dgrad': 1, 'conv_wgrad': 2, 'conv_wgrad_reduce': 3, 'conv_prep': 4,
-    'bn_fwd_reduce': 5, 'bn_fwd_apply': 6, 'bn_bwd_reduce': 7, 'bn_bwd_apply': 8,
+    'bn_fwd_reduce': 5, 'bn_fwd_apply': 6, 'bn_bwd_reduce': 7, 'bn_bwd_apply': 8, 'maxpool_fwd': 9, 'maxpool_bwd': 10,
 }
 
 

@@ -1,11 +1,13 @@
 """The hot-path autograd functions with the reference's names, arguments and error behaviour
 (``src/tortto/autograd/grad_nn.py``): ``Convolution`` (:684-734), ``TransposedConvolution``
-(:737-779), ``BatchNorm`` (:907-989) and ``Relu`` (:33-69).
+(:737-779), ``BatchNorm`` (:907-989), ``Relu`` (:33-69), ``LeakyRelu`` (:71-95) and
+``MaxPool2DWithIndices`` (:826-864).
 
 Where the reference evaluates NumPy/CuPy expressions, these call ``libtortto_hip.so`` through
 ``pytortto_amd.ops``.  Only device tensors (``hiparray``) are computed here: host tensors stay
 with tortto's own NumPy path, and are refused rather than silently computed some other way.
 """
+import math
 from math import prod
 
 import numpy as np
@@ -189,3 +191,96 @@ class Relu(Function):
         if yd0.__class__ is hiparray:
             return ops.relu_bwd(gd0, yd0)
         return gd0 * (yd0 > 0)
+
+
+class LeakyRelu(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, = inputs
+        xd0 = xt0.data
+        inplace = params['inplace']
+        negative_slope = params['negative_slope']
+        if xd0.__class__ is hiparray:
+            if inplace:
+                inplace_precheck(xt0)
+                ops.leaky_relu_fwd(xd0, negative_slope, out=xd0)
+                yt0 = inplace_update(xt0, ctx)
+            else:
+                yt0 = build_links(ops.leaky_relu_fwd(xd0, negative_slope), grad_fn=ctx)
+        elif inplace:
+            inplace_precheck(xt0)
+            np.maximum(xd0 * negative_slope, xd0, out=xd0)
+            yt0 = inplace_update(xt0, ctx)
+        else:
+            yt0 = build_links(np.maximum(xd0 * negative_slope, xd0), grad_fn=ctx)
+        ctx.save_for_backward(xt0)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        # the reference scales the incoming gradient array in place and hands it on (:94-95)
+        gd0, = grad_outputs
+        xd0, = ctx.saved_tensors
+        negative_slope = ctx.params['negative_slope']
+        if xd0.__class__ is hiparray:
+            return ops.leaky_relu_bwd(gd0, xd0, negative_slope, out=gd0)
+        gd0[xd0 < 0] *= negative_slope
+        return gd0
+
+
+def pool_output_size(size, k, stride, pad, dil, ceil_mode):
+    """Window count along one axis (``_sliding_window_view``, :565-579): floor rule, or the ceil
+    rule less the last window when it would start beyond the input and its leading padding."""
+    span = size + 2 * pad - dil * (k - 1) - 1
+    if not ceil_mode:
+        return math.floor(span / stride + 1)
+    out = math.ceil(span / stride + 1)
+    extra = (out - 1) * stride - span
+    if extra + pad >= (k - 1) * dil + 1:
+        out -= 1
+    return out
+
+
+def _reference_pos(tap, kw):
+    """The index tuple the reference returns for ``return_indices=True`` (:787-803), as host arrays:
+    aranges over (N, P, Q, C) and, per window, the kernel row and kernel column of its maximum."""
+    t = tap.get().reshape((-1,) + tap.shape[-3:])      # [N,C,P,Q]; a 3-D input counts as N = 1
+    t = np.moveaxis(t, 1, -1).astype(np.int64)         # [N,P,Q,C]
+    n, p, q, c = t.shape
+    return (np.arange(n)[:, None, None, None], np.arange(p)[None, :, None, None],
+            np.arange(q)[None, None, :, None], np.arange(c)[None, None, None, :], t // kw, t % kw)
+
+
+class MaxPool2DWithIndices(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, = inputs
+        xd0 = xt0.data
+        kernel_size = params['kernel_size']
+        stride = params['stride']
+        padding = params['padding']
+        dilation = params['dilation']
+        ceil_mode = params['ceil_mode']
+        return_indices = params['return_indices']
+        if padding[0] * 2 > kernel_size[0] or padding[1] * 2 > kernel_size[1]:
+            raise RuntimeError(f'pad should be smaller than or equal to half of kernel size, '
+                               f'but got padW = {padding[1]}, padH = {padding[0]}, kW = {kernel_size[1]}, '
+                               f'kH = {kernel_size[0]}')
+        if xd0.ndim != 3 and xd0.ndim != 4:
+            raise RuntimeError('non-empty 3D or 4D (batch mode) tensor expected for input')
+        _device_only('max_pool2d', xd0)
+        out_hw = tuple(pool_output_size(xd0.shape[-2 + a], kernel_size[a], stride[a], padding[a], dilation[a],
+                                        ceil_mode) for a in (0, 1))
+        yd0, tap = ops.maxpool2d_fwd(xd0, out_hw, kernel_size, stride, padding, dilation)
+        yt0 = build_links(yd0, grad_fn=ctx)
+        ctx.save_for_backward(xt0)
+        ctx.params['pos'] = tap
+        return (yt0, _reference_pos(tap, kernel_size[1])) if return_indices else yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, *_ = grad_outputs
+        xd0, = ctx.saved_tensors
+        p = ctx.params
+        return ops.maxpool2d_bwd(gd0, p['pos'], xd0.shape[-2:], p['kernel_size'], p['stride'], p['padding'],
+                                 p['dilation'])

@@ -1,4 +1,4 @@
-// Elementwise glue kernels (ReLU, residual add, gradient accumulation, fill): HBM-bound,
+// Elementwise glue kernels (ReLU, LeakyReLU, residual add, gradient accumulation, fill): HBM-bound,
 // float4 grid-stride loops with a scalar tail.
 #include "tt_common.h"
 
@@ -6,11 +6,17 @@ namespace {
 
 constexpr int kThreads = 256;
 
-enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill };
+enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill, kLeakyRelu, kLeakyReluBwd };
 
 template <int OP>
 __device__ __forceinline__ float apply1(float a, float b, float alpha) {
-  if (OP == kRelu) return fmaxf(a, 0.f);
+  // NumPy's maximum propagates NaN (src/tortto/autograd/grad_nn.py:56), fmaxf would drop it
+  if (OP == kRelu) return (a > 0.f || a != a) ? a : 0.f;
+  if (OP == kLeakyRelu) {                         // maximum(x * slope, x), grad_nn.py:85
+    const float t = a * alpha;
+    return (t > a || t != t) ? t : a;
+  }
+  if (OP == kLeakyReluBwd) return b < 0.f ? a * alpha : a;   // a = dy, b = x: g[x < 0] *= slope, grad_nn.py:94
   if (OP == kReluBwd) return b > 0.f ? a : 0.f;  // a = dy, b = y
   if (OP == kAdd) return a + b;
   if (OP == kAxpy) return fmaf(alpha, a, b);      // a = v, b = acc
@@ -21,7 +27,7 @@ template <int OP>
 __global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a, const float* __restrict__ b,
                                                     float* __restrict__ out, float alpha, size_t n) {
   constexpr bool kUseA = OP != kFill;
-  constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy;
+  constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy || OP == kLeakyReluBwd;
   const size_t n4 = n >> 2;
   const size_t stride = (size_t)gridDim.x * kThreads;
   for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
@@ -59,6 +65,12 @@ extern "C" {
 int tt_relu_fwd_f32(const float* x, float* y, size_t n) { return run<kRelu>("tt_relu_fwd_f32", x, nullptr, y, 0.f, n); }
 int tt_relu_bwd_f32(const float* dy, const float* y, float* dx, size_t n) {
   return run<kReluBwd>("tt_relu_bwd_f32", dy, y, dx, 0.f, n);
+}
+int tt_leaky_relu_fwd_f32(const float* x, float* y, float negative_slope, size_t n) {
+  return run<kLeakyRelu>("tt_leaky_relu_fwd_f32", x, nullptr, y, negative_slope, n);
+}
+int tt_leaky_relu_bwd_f32(const float* dy, const float* x, float* dx, float negative_slope, size_t n) {
+  return run<kLeakyReluBwd>("tt_leaky_relu_bwd_f32", dy, x, dx, negative_slope, n);
 }
 int tt_add_f32(const float* a, const float* b, float* out, size_t n) { return run<kAdd>("tt_add_f32", a, b, out, 0.f, n); }
 int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n) {

@@ -2,6 +2,8 @@ from .module import Module
 from .conv import Conv2d, ConvTranspose2d
 from .batchnorm import BatchNorm1d, BatchNorm2d, BatchNorm3d
 from .container import Sequential
-from .activation import ReLU
+from .activation import LeakyReLU, ReLU
+from .pooling import MaxPool2d
 
-__all__ = ['Module', 'Conv2d', 'ConvTranspose2d', 'BatchNorm1d', 'BatchNorm2d', 'BatchNorm3d', 'Sequential', 'ReLU']
+__all__ = ['Module', 'Conv2d', 'ConvTranspose2d', 'BatchNorm1d', 'BatchNorm2d', 'BatchNorm3d', 'Sequential', 'ReLU',
+           'LeakyReLU', 'MaxPool2d']

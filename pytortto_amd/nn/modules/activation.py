@@ -1,4 +1,4 @@
-"""``ReLU`` (``src/tortto/nn/modules/activation.py:24-34``)."""
+"""``ReLU`` and ``LeakyReLU`` (``src/tortto/nn/modules/activation.py:24-48``)."""
 from .. import functional as F
 from .module import Module
 
@@ -13,3 +13,17 @@ class ReLU(Module):
 
     def extra_repr(self):
         return 'inplace=True' if self.inplace else ''
+
+
+class LeakyReLU(Module):
+    def __init__(self, negative_slope=1e-2, inplace=False):
+        super().__init__()
+        self.negative_slope = negative_slope
+        self.inplace = inplace
+
+    def forward(self, tensor):
+        return F.leaky_relu(tensor, self.negative_slope, self.inplace)
+
+    def extra_repr(self):
+        inplace_str = ', inplace=True' if self.inplace else ''
+        return f'negative_slope={self.negative_slope}{inplace_str}'

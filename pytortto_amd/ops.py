@@ -5,6 +5,7 @@ Shape bookkeeping and output allocation happen here; all arithmetic happens in
 stands in for (paths relative to the reference's ``src/tortto/``).
 """
 import math
+from math import prod
 
 import numpy as np
 
@@ -145,6 +146,20 @@ def relu_bwd(dy, y):
     return dx
 
 
+def leaky_relu_fwd(x, negative_slope, out=None):
+    _f32(x)
+    y = hiparray.empty(x.shape) if out is None else out
+    _hip.call('tt_leaky_relu_fwd_f32', x.ptr, y.ptr, float(negative_slope), x.size)
+    return y
+
+
+def leaky_relu_bwd(dy, x, negative_slope, out=None):
+    _f32(dy, x)
+    dx = hiparray.empty(x.shape) if out is None else out
+    _hip.call('tt_leaky_relu_bwd_f32', dy.ptr, x.ptr, dx.ptr, float(negative_slope), x.size)
+    return dx
+
+
 def add(a, b):
     _f32(a, b)
     if a.shape != b.shape:
@@ -152,3 +167,38 @@ def add(a, b):
     out = hiparray.empty(a.shape)
     _hip.call('tt_add_f32', a.ptr, b.ptr, out.ptr, a.size)
     return out
+
+
+# ---- MaxPool2d -------------------------------------------------------------------------------------
+
+def _pool_dims(x):
+    if x.ndim not in (3, 4):
+        raise ValueError(f'max pooling needs [N,C,H,W] or [C,H,W] planes, got shape {x.shape}')
+    return prod(x.shape[:-2]), x.shape[-2], x.shape[-1]
+
+
+def maxpool2d_fwd(x, out_hw, kernel_size, stride, padding, dilation):
+    """(y, tap): maxima over the -inf padded windows and, per output, the winning tap as
+    kernel_row * kw + kernel_column (``_max_pool2d``, grad_nn.py:784-808)."""
+    _f32(x)
+    nc, h, w = _pool_dims(x)
+    p, q = out_hw
+    y = hiparray.empty(x.shape[:-2] + (p, q))
+    tap = hiparray.empty(x.shape[:-2] + (p, q), np.int32)
+    _hip.call('tt_maxpool2d_fwd_f32', x.ptr, y.ptr, tap.ptr, nc, h, w, p, q, *kernel_size, *stride, *padding,
+              *dilation)
+    return y, tap
+
+
+def maxpool2d_bwd(dy, tap, in_hw, kernel_size, stride, padding, dilation):
+    """dx: every output gradient assigned to its window's arg-max pixel, the last window in
+    (p, q) order winning where several chose the same pixel (``_max_pool2d_backward``, :811-824)."""
+    _f32(dy)
+    if tap.dtype != np.int32 or tap.shape != dy.shape:
+        raise ValueError('maxpool2d_bwd: `tap` must be the int32 array the forward returned')
+    nc, p, q = _pool_dims(dy)
+    h, w = in_hw
+    dx = hiparray.empty(dy.shape[:-2] + (h, w))
+    _hip.call('tt_maxpool2d_bwd_f32', dy.ptr, tap.ptr, dx.ptr, nc, h, w, p, q, *kernel_size, *stride, *padding,
+              *dilation)
+    return dx

@@ -100,3 +100,49 @@ def conv_transpose2d_def(x, w, b, stride, padding, output_padding, dilation, gro
     if b is not None:
         y += b.astype(np.float64)[None, :, None, None]
     return y
+
+
+def max_pool2d_def(x, kernel_size, stride, padding, dilation, out_hw):
+    """(y, arg): window maxima over the -inf padded input, first maximum in (row, column)
+    order; arg[n,c,p,q] = (input row, input column) of the chosen element, or None when it
+    lies in the padding."""
+    n, c, h, w = x.shape
+    (kh, kw), (sh, sw), (ph, pw), (dh, dw) = kernel_size, stride, padding, dilation
+    p_out, q_out = out_hw
+    y = np.empty((n, c, p_out, q_out), x.dtype)
+    arg = np.empty((n, c, p_out, q_out), object)
+    for nn in range(n):
+        for cc in range(c):
+            for p in range(p_out):
+                for q in range(q_out):
+                    best, where = -np.inf, None
+                    first = True
+                    for i in range(kh):
+                        for j in range(kw):
+                            hh, ww = p * sh - ph + i * dh, q * sw - pw + j * dw
+                            inside = 0 <= hh < h and 0 <= ww < w
+                            v = x[nn, cc, hh, ww] if inside else -np.inf
+                            if first or v > best:
+                                best, where = v, ((hh, ww) if inside else None)
+                            first = False
+                    y[nn, cc, p, q] = best
+                    arg[nn, cc, p, q] = where
+    return y, arg
+
+
+def max_pool2d_backward_def(x_shape, grad, arg, accumulate=False):
+    """Visit the windows in (n, c, p, q) order and write (or add) each gradient at its arg-max."""
+    dx = np.zeros(x_shape, grad.dtype)
+    n, c, p_out, q_out = grad.shape
+    for nn in range(n):
+        for cc in range(c):
+            for p in range(p_out):
+                for q in range(q_out):
+                    where = arg[nn, cc, p, q]
+                    if where is None:
+                        continue
+                    if accumulate:
+                        dx[nn, cc, where[0], where[1]] += grad[nn, cc, p, q]
+                    else:
+                        dx[nn, cc, where[0], where[1]] = grad[nn, cc, p, q]
+    return dx

@@ -26,3 +26,16 @@ CONVT_CASES = [
     (2, 4, 4, 5, 4, 3, 3, (2, 2), (0, 0), (1, 0), (2, 2), 1),   # gcd(stride, dilation) = 2
     (1, 2, 3, 3, 2, 2, 2, (3, 3), (0, 0), (2, 2), (1, 1), 1),   # stride > kernel: holes in the output
 ]
+
+# (N, C, H, W, kernel, stride, padding, dilation, ceil_mode)
+POOL_CASES = [
+    (2, 3, 8, 8, (2, 2), (2, 2), (0, 0), (1, 1), False),      # non-overlapping
+    (2, 3, 9, 7, (3, 3), (2, 2), (1, 1), (1, 1), False),      # ResNet stem geometry: overlapping windows
+    (1, 4, 12, 12, (3, 3), (2, 2), (1, 1), (1, 1), True),     # ceil_mode adds a partial window
+    (2, 2, 10, 11, (3, 2), (1, 2), (1, 0), (1, 1), False),    # stride 1 in H: heavy overlap
+    (2, 2, 11, 10, (2, 3), (2, 1), (1, 1), (2, 2), False),    # dilation
+    (1, 3, 7, 7, (3, 3), (3, 3), (0, 0), (1, 1), True),       # ceil_mode, window hanging over the edge
+    (1, 2, 6, 6, (2, 2), (2, 2), (1, 1), (1, 1), True),       # ceil_mode whose last window is dropped
+    (3, 1, 5, 9, (5, 3), (1, 3), (2, 1), (1, 1), False),      # tall kernel
+    (2, 2, 8, 8, (2, 2), (3, 3), (0, 0), (1, 1), False),      # stride > kernel: uncovered pixels
+]
