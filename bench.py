@@ -130,6 +130,18 @@ def profiled_steps(hip, step, steps):
     return prof
 
 
+def cpu_baseline_pool(batch):
+    """(bytes counted, seconds) of the oracle's MaxPool2d forward + backward."""
+    import oracle
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((batch, 64, 112, 112), dtype=np.float32)
+    t0 = time.perf_counter()
+    y, pos = oracle.max_pool2d(x, (3, 3), (2, 2), (1, 1))
+    oracle.max_pool2d_backward(x.shape, y, pos, (3, 3), (2, 2), (1, 1))
+    sec = time.perf_counter() - t0
+    return 2 * (x.nbytes + 2 * y.nbytes), sec
+
+
 def cpu_threads():
     try:
         from threadpoolctl import threadpool_info
@@ -193,6 +205,7 @@ def main():
         sys.exit(2)
 
     from pytortto_amd import _hip
+    from pytortto_amd.xparray import hiparray
     from pytortto_amd._paths import LIB_PATH
     if not os.path.exists(LIB_PATH):
         from pytortto_amd.build import build_library
@@ -246,6 +259,42 @@ def main():
     n_ba, ms_ba = bprof['bn_bwd_apply']
     bwd_apply_gbs = sum(3 * b.bytes for b in bns) * args.steps / (ms_ba * 1e-3) / 1e9
     del bns
+    call('tt_empty_cache')
+
+    # ---- rows either side of the path: MaxPool2d (ResNet-50 stem pooling) and the activations ---
+    pool_shape, pool_args = (BATCH, 64, 112, 112), (3, 3, 2, 2, 1, 1, 1, 1)
+    px = hiparray(rng.standard_normal(pool_shape, dtype=np.float32))
+    py = hiparray.empty((BATCH, 64, 56, 56))
+    ptap = hiparray.empty((BATCH, 64, 56, 56), np.int32)
+    pdx = hiparray.empty(pool_shape)
+    pool_dims = (BATCH * 64, 112, 112, 56, 56)
+
+    def pool_step():
+        call('tt_maxpool2d_fwd_f32', px.ptr, py.ptr, ptap.ptr, *pool_dims, *pool_args)
+        call('tt_maxpool2d_bwd_f32', py.ptr, ptap.ptr, pdx.ptr, *pool_dims, *pool_args)
+
+    pool_ms, _ = timed_steps(_hip, pool_step, args.steps, args.warmup)
+    pprof = profiled_steps(_hip, pool_step, args.steps)
+    # algorithmic bytes: forward reads x, writes y and the int32 taps; backward reads dy and taps, writes dx
+    pool_fwd_bytes = px.nbytes + py.nbytes + ptap.nbytes
+    pool_bytes = 2 * pool_fwd_bytes
+    n_pb, ms_pb = pprof['maxpool_bwd']
+    n_pf, ms_pf = pprof['maxpool_fwd']
+    pool_bwd_gbs = pool_fwd_bytes * n_pb / (ms_pb * 1e-3) / 1e9
+    act = {}
+    for name, fn, nbytes in (
+            ('relu_fwd', lambda: call('tt_relu_fwd_f32', px.ptr, pdx.ptr, px.size), 2 * px.nbytes),
+            ('relu_bwd', lambda: call('tt_relu_bwd_f32', px.ptr, pdx.ptr, pdx.ptr, px.size), 3 * px.nbytes),
+            ('leaky_relu_fwd', lambda: call('tt_leaky_relu_fwd_f32', px.ptr, pdx.ptr, 0.2, px.size), 2 * px.nbytes),
+            ('add', lambda: call('tt_add_f32', px.ptr, pdx.ptr, pdx.ptr, px.size), 3 * px.nbytes)):
+        ms, _ = timed_steps(_hip, fn, args.steps, 2)
+        act[name] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+    cpu_pool = None
+    if not args.no_cpu_baseline:
+        nb, sec = cpu_baseline_pool(32)
+        cpu_pool = {'value': round(nb / sec / 1e9, 3), 'unit': 'GB/s', 'cores': 1, 'kind': 'port',
+                    'sample': f'oracle MaxPool2d fwd+bwd at [32,64,112,112] ({nb / 1e9:.2f} GB counted, {sec:.1f} s)'}
+    del px, py, ptap, pdx
     call('tt_empty_cache')
 
     # ---- what the device sustains on the two bounding resources, measured in this run ----------
@@ -304,6 +353,19 @@ def main():
                             'avg_launch_ms': round(ms_ba / max(1, n_ba), 5)},
                'kernels_ms_per_step': bn_kernel_ms,
                'cpu_baseline': cpu_bn},
+        'maxpool': {'metric': 'MaxPool2d fwd+bwd GB/s', 'value': round(pool_bytes / (pool_ms * 1e-3) / 1e9, 1),
+                    'unit': 'GB/s', 'ms_per_step': round(pool_ms, 4),
+                    'pct_of_peak': round(100 * pool_bytes / (pool_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 1),
+                    'config': {'workload': 'MaxPool2d(3, stride 2, padding 1) fwd+bwd fp32 NCHW at [64,64,112,112] '
+                                           '(ResNet-50 stem pooling); bytes: x + y + int32 taps, both ways'},
+                    'roofline': {'bound': 'hbm', 'kernel': 'maxpool_bwd_scatter (reads dy, taps; writes dx)',
+                                 'achieved': round(pool_bwd_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                                 'frac': round(pool_bwd_gbs / PEAK_HBM_GBS, 4), 'traffic': None,
+                                 'avg_launch_ms': round(ms_pb / max(1, n_pb), 5)},
+                    'kernels_ms_per_step': {'maxpool_fwd': round(ms_pf / max(1, n_pf), 4),
+                                            'maxpool_bwd': round(ms_pb / max(1, n_pb), 4)},
+                    'elementwise_gbs_at_same_size': act,
+                    'cpu_baseline': cpu_pool},
     }
     print(json.dumps(out))
 

@@ -42,6 +42,14 @@ def test_max_pool_resnet_stem_shape_reduced_batch():
     _run_pool((2, 16, 113, 57, (3, 3), (2, 2), (1, 1), (1, 1), True), seed=6, ties=True)
 
 
+def test_max_pool_rows_too_wide_for_the_lds_stage():
+    # three input rows of 1500 (forward) / two gradient rows of 1100 (backward) exceed the staged
+    # span: both passes take the direct kernels
+    _run_pool((1, 2, 8, 1500, (3, 3), (2, 2), (1, 1), (1, 1), False), seed=10, ties=True)
+    _run_pool((1, 1, 6, 2200, (3, 3), (2, 2), (1, 1), (1, 1), False), seed=11, ties=False)
+    _run_pool((1, 2, 40, 700, (5, 2), (1, 1), (2, 1), (1, 1), False), seed=12, ties=True)   # one output row per block
+
+
 def test_max_pool_full_size_properties():
     """[64,64,112,112], 3x3 stride 2 padding 1 (the ResNet-50 stem pooling): with dy = y every
     assigned gradient equals the input at that pixel, each window's maximum is found in the
