@@ -160,6 +160,36 @@ int tt_maxpool2d_fwd_f32(const float* x, float* y, int* tap, int NC, int H, int 
 int tt_maxpool2d_bwd_f32(const float* dy, const int* tap, float* dx, int NC, int H, int W, int P, int Q,
                          int kh, int kw, int sh, int sw, int ph, int pw, int dh, int dw);
 
+/* ---- classifier head: spatial mean, Linear, LogSoftmax, NLLLoss ------------------------------- */
+
+/* y[r] = mean(x[r, 0..L)) and its gradient dx[r, i] = g[r] / L: `Mean` over trailing dimensions
+ * (autograd/grad_fcn.py:1058-1093; `tt.mean(x, (-1, -2), True)` in the ResNet examples). */
+int tt_mean_rows_f32(const float* x, float* y, int R, int L);
+int tt_mean_rows_bwd_f32(const float* g, float* dx, int R, int L);
+/* y[c, r] = x[r, c]: `Transpose` of a matrix, materialised (grad_fcn.py:752-771; `weight.T` in
+ * nn/functional.py:59).  The matrix products of `Mm` (grad_fcn.py:907-932) need no entry point of
+ * their own: A[M,K] @ B[K,N] is tt_conv2d_fwd_f32 on the image B = [1, K, 1, N] with the 1x1
+ * weights A = [M, K, 1, 1]; G @ B^T is tt_conv2d_wgrad_f32 and A^T @ G is tt_conv2d_dgrad_f32 of
+ * the same geometry. */
+int tt_transpose2d_f32(const float* x, float* y, int R, int C);
+/* out[r, c] = a[r, c] + v[c]: `Add` with the bias broadcast over rows (grad_fcn.py:177-203;
+ * nn/functional.py:59); the bias gradient is tt_channel_sum_f32(g, db, R, C, 1). */
+int tt_add_rowvec_f32(const float* a, const float* v, float* out, int R, int C);
+/* Row-wise y = (x - max) - log(sum(exp(x - max))) and dx = g - sum(g) * exp(y)
+ * (autograd/grad_nn.py:373-392).  A NaN in a row makes the whole row NaN, as NumPy's max does. */
+int tt_log_softmax_fwd_f32(const float* x, float* y, int R, int C);
+int tt_log_softmax_bwd_f32(const float* g, const float* y, float* dx, int R, int C);
+/* NllLoss on logp[R, C] with int64 targets (autograd/grad_nn.py:287-349).  weight: per-class
+ * weights or NULL; ignore_index acts only when >= 0, as in the reference (:301-305).
+ * reduction: 0 none (out[R]), 1 sum, 2 mean (out[1]); `count` (device, 1 float) receives the
+ * mean's divisor: R without weights, else the number of rows with non-zero weight (:315-319).
+ * The backward takes the same `count`; g is [R] for reduction none, else one value.  Targets
+ * outside [0, C) raise IndexError in the reference; here such rows contribute nothing. */
+int tt_nll_loss_fwd_f32(const float* logp, const long long* target, const float* weight, float* out,
+                        float* count, int R, int C, long long ignore_index, int reduction);
+int tt_nll_loss_bwd_f32(const float* g, const long long* target, const float* weight, const float* count,
+                        float* dlogp, int R, int C, long long ignore_index, int reduction);
+
 /* ---- elementwise glue so whole stacks stay on the device ----------------------------------- */
 
 /* y = max(x, 0) (autograd/grad_nn.py:33-69); dx = dy * (y > 0). */

@@ -23,6 +23,9 @@ publishes no golden vectors for this path):
                         torch CPU ``F.max_pool2d`` (forward always; backward where windows do
                         not overlap, so that assignment and summation coincide)
 * ``relu*/leaky_relu*`` closed forms on signs / zero / NaN, torch CPU with autograd
+* ``mean_*``, ``mm_*``, ``linear_*``, ``log_softmax_*``, ``nll_loss_*``
+                        torch CPU functions with autograd (weights, ignore_index, reductions),
+                        closed forms (normalisation, zero-sum gradient rows, g / count)
 
 The checks live in ``tests/test_oracle_*.py``.
 """
@@ -32,6 +35,8 @@ from .conv import (conv2d, conv2d_backward_w, conv2d_backward_x, conv_output_siz
 from .batchnorm import batch_norm_forward, batch_norm_backward
 from .nninit import conv_parameters, bn_affine_c4
 from .pool import max_pool2d, max_pool2d_backward, pool_output_size
+from .head import (mean_forward, mean_backward, mm_forward, mm_backward, linear_forward, linear_backward,
+                   log_softmax_forward, log_softmax_backward, nll_loss_forward, nll_loss_backward)
 from .activation import relu_forward, relu_backward, leaky_relu_forward, leaky_relu_backward
 
 __all__ = [
@@ -41,4 +46,6 @@ __all__ = [
     'batch_norm_forward', 'batch_norm_backward', 'conv_parameters', 'bn_affine_c4',
     'max_pool2d', 'max_pool2d_backward', 'pool_output_size',
     'relu_forward', 'relu_backward', 'leaky_relu_forward', 'leaky_relu_backward',
+    'mean_forward', 'mean_backward', 'mm_forward', 'mm_backward', 'linear_forward', 'linear_backward',
+    'log_softmax_forward', 'log_softmax_backward', 'nll_loss_forward', 'nll_loss_backward',
 ]

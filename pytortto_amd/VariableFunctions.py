@@ -41,3 +41,59 @@ def tensor(data, requires_grad=False, dtype=None, copy=True, **kwargs):
     if dtype is None:
         dtype = getattr(data, 'dtype', float32)
     return Tensor(data, requires_grad=requires_grad, dtype=dtype, copy=copy, **kwargs)
+
+
+# ---- the few array functions the classifier head of the ResNet examples uses ----------------------
+
+def transpose(input, dim0, dim1):
+    return input.transpose(dim0, dim1)
+
+
+swapaxes = transpose
+swapdims = transpose
+
+
+def mean(input, dim=None, keepdim=False):
+    return input.mean(dim, keepdim)
+
+
+def flatten(x, start_dim=0, end_dim=-1):
+    """VariableFunctions.py:108-127."""
+    shape = x.shape
+    if end_dim < 0:
+        end_dim = len(shape) + end_dim
+    end_dim += 1
+    if start_dim < 0:
+        start_dim = len(shape) + start_dim
+    if start_dim >= end_dim:
+        raise RuntimeError('flatten() has invalid args: start_dim cannot come after end_dim')
+    newshape = shape[:start_dim]
+    if start_dim != end_dim:
+        newshape += (-1,)
+    if end_dim < len(shape):
+        newshape += shape[end_dim:]
+    if len(newshape) != len(shape):
+        return x.view(newshape)
+    return x
+
+
+def mm(input, mat2):
+    from .autograd.grad_fcn import Mm
+    return Mm.apply(input, mat2)
+
+
+def matmul(input, other):
+    """VariableFunctions.py:365-396, for the cases the head needs: matrix @ matrix, and a tensor with
+    leading dimensions @ matrix (collapsed to a matrix product and restored)."""
+    from .autograd.grad_fcn import Mm, View
+    if input.ndim == 0 or other.ndim == 0:
+        raise RuntimeError(f'both arguments to matmul need to be at least 1D, but they are {input.ndim}D and '
+                           f'{other.ndim}D')
+    if input.ndim == 2 and other.ndim == 2:
+        return Mm.apply(input, other)
+    if other.ndim == 2 and input.ndim > 2:
+        leading_dims = input.shape[:-1]
+        input = View.apply(input, shape=(-1, input.shape[-1]))
+        result = Mm.apply(input, other)
+        return View.apply(result, shape=(*leading_dims, result.shape[-1]))
+    raise NotImplementedError(f'matmul of a {input.ndim}D and a {other.ndim}D tensor is outside this build')

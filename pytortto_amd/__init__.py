@@ -12,9 +12,11 @@ import numpy as np
 
 from .xparray import nparray, hiparray
 from .tensor import Tensor, float16, float32, float64, int16, int32, int64
-from .VariableFunctions import manual_seed, empty, zeros, ones, randn, tensor
+from .VariableFunctions import (manual_seed, empty, zeros, ones, randn, tensor, transpose, swapaxes, swapdims,
+                                mean, flatten, mm, matmul)
 from .autograd import (no_grad, enable_grad, set_grad_enabled, is_grad_enabled, Function, AccumulateGrad,
-                       ToCopy, Add, Convolution, TransposedConvolution, BatchNorm, Relu)
+                       ToCopy, Add, Convolution, TransposedConvolution, BatchNorm, Relu, LeakyRelu,
+                       MaxPool2DWithIndices, LogSoftmax, NllLoss, View, Transpose, Mm, Mean)
 from . import nn
 from . import _hip
 

@@ -47,6 +47,14 @@ PROTOTYPES = {
     'tt_leaky_relu_bwd_f32': [_P, _P, _P, c_float, c_size_t],
     'tt_maxpool2d_fwd_f32': [_P, _P, _P] + [_I] * 13,
     'tt_maxpool2d_bwd_f32': [_P, _P, _P] + [_I] * 13,
+    'tt_mean_rows_f32': [_P, _P, _I, _I],
+    'tt_mean_rows_bwd_f32': [_P, _P, _I, _I],
+    'tt_transpose2d_f32': [_P, _P, _I, _I],
+    'tt_add_rowvec_f32': [_P, _P, _P, _I, _I],
+    'tt_log_softmax_fwd_f32': [_P, _P, _I, _I],
+    'tt_log_softmax_bwd_f32': [_P, _P, _P, _I, _I],
+    'tt_nll_loss_fwd_f32': [_P, _P, _P, _P, _P, _I, _I, ctypes.c_longlong, _I],
+    'tt_nll_loss_bwd_f32': [_P, _P, _P, _P, _P, _I, _I, ctypes.c_longlong, _I],
     'tt_add_f32': [_P, _P, _P, c_size_t],
     'tt_axpy_f32': [c_float, _P, _P, c_size_t],
     'tt_fill_f32': [_P, c_float, c_size_t],

@@ -1,7 +1,7 @@
 """The hot-path autograd functions with the reference's names, arguments and error behaviour
 (``src/tortto/autograd/grad_nn.py``): ``Convolution`` (:684-734), ``TransposedConvolution``
 (:737-779), ``BatchNorm`` (:907-989), ``Relu`` (:33-69), ``LeakyRelu`` (:71-95) and
-``MaxPool2DWithIndices`` (:826-864).
+``MaxPool2DWithIndices`` (:826-864), ``LogSoftmax`` (:373-392), ``NllLoss`` (:287-349).
 
 Where the reference evaluates NumPy/CuPy expressions, these call ``libtortto_hip.so`` through
 ``pytortto_amd.ops``.  Only device tensors (``hiparray``) are computed here: host tensors stay
@@ -284,3 +284,59 @@ class MaxPool2DWithIndices(Function):
         p = ctx.params
         return ops.maxpool2d_bwd(gd0, p['pos'], xd0.shape[-2:], p['kernel_size'], p['stride'], p['padding'],
                                  p['dilation'])
+
+
+class LogSoftmax(Function):
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, = inputs
+        xd0 = xt0.data
+        dim = params['dim']
+        if xd0.__class__ is hiparray:
+            if dim % xd0.ndim != xd0.ndim - 1:
+                raise RuntimeError(f'device log_softmax reduces the last dimension only, got dim={dim} for shape '
+                                   f'{xd0.shape}')
+            yd0 = ops.log_softmax_fwd(xd0)
+        else:
+            aug = xd0 - np.max(xd0, axis=dim, keepdims=True)
+            yd0 = aug - np.log(np.sum(np.exp(aug), axis=dim, keepdims=True))
+        yt0 = build_links(yd0, grad_fn=ctx)
+        ctx.save_for_backward(yt0)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        dim = ctx.params['dim']
+        yd0, = ctx.saved_tensors
+        if yd0.__class__ is hiparray:
+            return ops.log_softmax_bwd(gd0, yd0)
+        return gd0 - gd0.sum(axis=dim, keepdims=True) * np.exp(yd0)
+
+
+class NllLoss(Function):
+    """Device tensors only: logp [N, C] with an int64 target [N] (the classification head)."""
+
+    @staticmethod
+    def forward(ctx, *inputs, **params):
+        xt0, = inputs
+        xt1 = params['target']
+        xd0, xd1 = xt0.data, xt1.data
+        reduction = params['reduction']
+        weight = params['weight']
+        ignore_index = params['ignore_index']
+        _device_only('nll_loss', xd0)
+        if xd1.__class__ is not hiparray or (weight is not None and weight.data.__class__ is not hiparray):
+            raise RuntimeError('Expected all tensors to be on the same device')
+        yd0, count = ops.nll_loss_fwd(xd0, xd1, None if weight is None else weight.data, ignore_index, reduction)
+        ctx.params['N'] = count
+        yt0 = build_links(yd0, grad_fn=ctx)
+        ctx.save_for_backward(xt0, xt1, weight)
+        return yt0
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        gd0, = grad_outputs
+        p = ctx.params
+        xd0, xd1, w = ctx.saved_tensors
+        return ops.nll_loss_bwd(gd0, xd0.shape, xd1, w, p['N'], p['ignore_index'], p['reduction'])

@@ -1,4 +1,4 @@
-"""``ReLU`` and ``LeakyReLU`` (``src/tortto/nn/modules/activation.py:24-48``)."""
+"""``ReLU``, ``LeakyReLU`` and ``LogSoftmax`` (``src/tortto/nn/modules/activation.py:24-48``, ``:75-84``)."""
 from .. import functional as F
 from .module import Module
 
@@ -27,3 +27,15 @@ class LeakyReLU(Module):
     def extra_repr(self):
         inplace_str = ', inplace=True' if self.inplace else ''
         return f'negative_slope={self.negative_slope}{inplace_str}'
+
+
+class LogSoftmax(Module):
+    def __init__(self, dim):
+        super().__init__()
+        self.dim = dim
+
+    def forward(self, tensor):
+        return F.log_softmax(tensor, self.dim)
+
+    def extra_repr(self):
+        return f'dim={self.dim}'

@@ -202,3 +202,123 @@ def maxpool2d_bwd(dy, tap, in_hw, kernel_size, stride, padding, dilation):
     _hip.call('tt_maxpool2d_bwd_f32', dy.ptr, tap.ptr, dx.ptr, nc, h, w, p, q, *kernel_size, *stride, *padding,
               *dilation)
     return dx
+
+
+# ---- classifier head -----------------------------------------------------------------------------
+
+def mean_trailing(x, k, keepdim):
+    """Mean over the last ``k`` dimensions (autograd/grad_fcn.py:1058-1067)."""
+    _f32(x)
+    lead, tail = x.shape[:-k], x.shape[-k:]
+    y = hiparray.empty(lead + ((1,) * k if keepdim else ()))
+    _hip.call('tt_mean_rows_f32', x.ptr, y.ptr, prod(lead), prod(tail))
+    return y
+
+
+def mean_trailing_bwd(g, x_shape, k):
+    """The gradient divided by the element count and repeated over the reduced dimensions
+    (grad_fcn.py:1069-1093); materialised, where the reference returns a stride-0 view."""
+    _f32(g)
+    dx = hiparray.empty(x_shape)
+    _hip.call('tt_mean_rows_bwd_f32', g.ptr, dx.ptr, prod(x_shape[:-k]), prod(x_shape[-k:]))
+    return dx
+
+
+def transpose2d(x):
+    _f32(x)
+    r, c = x.shape
+    y = hiparray.empty((c, r))
+    _hip.call('tt_transpose2d_f32', x.ptr, y.ptr, r, c)
+    return y
+
+
+_ONE = ((1, 1), (0, 0), (1, 1), 1)   # stride, padding, dilation, groups of a plain matrix product
+
+
+def mm(a, b):
+    """a[M,K] @ b[K,N] (grad_fcn.py:907-918) on the implicit-GEMM convolution kernel: b is the
+    image [1, K, 1, N], a the 1x1 weights [M, K, 1, 1]."""
+    (m, k), (k2, n) = a.shape, b.shape
+    if k != k2:
+        raise RuntimeError(f'mat1 and mat2 shapes cannot be multiplied ({m}x{k} and {k2}x{n})')
+    return conv2d_fwd(b.reshape((1, k, 1, n)), a.reshape((m, k, 1, 1)), None, *_ONE).reshape((m, n))
+
+
+def mm_grad_a(g, b):
+    """g[M,N] @ b[K,N].T (grad_fcn.py:927-928): the weight gradient of the same 1x1 geometry."""
+    (m, n), (k, _) = g.shape, b.shape
+    return conv2d_wgrad(b.reshape((1, k, 1, n)), g.reshape((1, m, 1, n)), (m, k, 1, 1), *_ONE).reshape((m, k))
+
+
+def mm_grad_b(a, g):
+    """a[M,K].T @ g[M,N] (grad_fcn.py:929-930): the input gradient of the same 1x1 geometry."""
+    (m, k), (_, n) = a.shape, g.shape
+    return conv2d_dgrad(g.reshape((1, m, 1, n)), a.reshape((m, k, 1, 1)), None, (1, n), *_ONE).reshape((k, n))
+
+
+def add_rowvec(a, v):
+    """a + v with ``v`` broadcast over the leading dimensions of ``a``."""
+    _f32(a, v)
+    c = v.size
+    out = hiparray.empty(a.shape)
+    _hip.call('tt_add_rowvec_f32', a.ptr, v.ptr, out.ptr, a.size // c, c)
+    return out
+
+
+def sum_rows(g, c):
+    """Sum over all but the trailing ``c`` elements: the gradient of a broadcast bias."""
+    _f32(g)
+    out = hiparray.empty((c,))
+    _hip.call('tt_channel_sum_f32', g.ptr, out.ptr, g.size // c, c, 1)
+    return out
+
+
+def log_softmax_fwd(x):
+    _f32(x)
+    c = x.shape[-1]
+    y = hiparray.empty(x.shape)
+    _hip.call('tt_log_softmax_fwd_f32', x.ptr, y.ptr, x.size // c, c)
+    return y
+
+
+def log_softmax_bwd(g, y):
+    _f32(g, y)
+    c = y.shape[-1]
+    dx = hiparray.empty(y.shape)
+    _hip.call('tt_log_softmax_bwd_f32', g.ptr, y.ptr, dx.ptr, y.size // c, c)
+    return dx
+
+
+_REDUCTIONS = {'none': 0, 'sum': 1, 'mean': 2}
+
+
+def _nll_args(logp, target, weight, reduction):
+    _f32(logp, weight)
+    if logp.ndim != 2 or target.shape != logp.shape[:1]:
+        raise RuntimeError(f'the device nll_loss takes logp [N, C] and target [N], got {logp.shape} and {target.shape}')
+    if target.dtype != np.int64:
+        raise RuntimeError(f'expected an int64 target, got {target.dtype}')
+    if reduction not in _REDUCTIONS:
+        raise ValueError(f'{reduction} is not a valid value for reduction')
+    return _REDUCTIONS[reduction]
+
+
+def nll_loss_fwd(logp, target, weight, ignore_index, reduction):
+    """(loss, count): grad_nn.py:287-327; ``count`` is the device-resident divisor of the mean."""
+    red = _nll_args(logp, target, weight, reduction)
+    r, c = logp.shape
+    out = hiparray.empty((r,) if red == 0 else ())
+    count = hiparray.empty((1,))
+    _hip.call('tt_nll_loss_fwd_f32', logp.ptr, target.ptr, _ptr(weight), out.ptr, count.ptr, r, c,
+              int(ignore_index), red)
+    return out, count
+
+
+def nll_loss_bwd(g, logp_shape, target, weight, count, ignore_index, reduction):
+    """grad_nn.py:329-349."""
+    _f32(g, weight)
+    r, c = logp_shape
+    dlogp = hiparray.empty(logp_shape)
+    _hip.call('tt_nll_loss_bwd_f32', g.ptr, target.ptr, _ptr(weight), count.ptr, dlogp.ptr, r, c,
+              int(ignore_index), _REDUCTIONS[reduction])
+    return dlogp

@@ -158,6 +158,39 @@ class Tensor:
         from .autograd.grad_fcn import Add
         return Add.apply(self, other)
 
+    def __matmul__(self, other):
+        from .VariableFunctions import matmul
+        return matmul(self, other)
+
+    @property
+    def T(self):
+        """tensor.py:56-60."""
+        if self.ndim != 2:
+            raise RuntimeError(f'x.T expects a tensor with 2 dimensions, but self is {self.ndim}D')
+        return self.transpose(1, 0)
+
+    def transpose(self, dim0, dim1):
+        from .autograd.grad_fcn import Transpose
+        return Transpose.apply(self, dim0=dim0, dim1=dim1)
+
+    swapaxes = transpose
+    swapdims = transpose
+
+    def mean(self, dim=None, keepdim=False):
+        from .autograd.grad_fcn import Mean
+        return Mean.apply(self, dim=dim, keepdim=keepdim)
+
+    def view(self, *shape):
+        """tensor.py:408-411."""
+        from .autograd.grad_fcn import View
+        if shape[0].__class__ is not int:
+            shape = shape[0]
+        return View.apply(self, shape=tuple(shape))
+
+    def flatten(self, start_dim=0, end_dim=-1):
+        from .VariableFunctions import flatten
+        return flatten(self, start_dim, end_dim)
+
     # ---- autograd ------------------------------------------------------------------------------
     def backward(self, gradient=None):
         """tensor.py:568-613."""

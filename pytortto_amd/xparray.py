@@ -87,9 +87,8 @@ class hiparray:
             self._buf, self._shape, self._dtype = _buf, tuple(_shape), np.dtype(dtype)
             self._version = _version if _version is not None else [0]
             return self
-        host = np.ascontiguousarray(np.asarray(input_array, dtype=dtype))
-        if host.ndim == 0:
-            host = host.reshape(())
+        given = np.asarray(input_array, dtype=dtype)
+        host = np.ascontiguousarray(given).reshape(given.shape)     # ascontiguousarray turns 0-d into 1-d
         self._shape = host.shape
         self._dtype = host.dtype
         self._version = [0]
