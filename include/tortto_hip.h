@@ -190,6 +190,22 @@ int tt_nll_loss_fwd_f32(const float* logp, const long long* target, const float*
 int tt_nll_loss_bwd_f32(const float* g, const long long* target, const float* weight, const float* count,
                         float* dlogp, int R, int C, long long ignore_index, int reduction);
 
+/* ---- optimiser steps (optim/_functional.py:4-119) ---------------------------------------------- */
+
+/* One SGD update of a parameter in place (_functional.py:4-22): d = grad (+ weight_decay * param);
+ * with momentum != 0, buf = d on the first step, else buf = buf * momentum + d * (1 - dampening),
+ * and d = buf (or d + buf * momentum with nesterov); param += d * (-lr).  Each product and sum is
+ * rounded to float32 separately, as NumPy evaluates the reference's expressions. */
+int tt_sgd_step_f32(float* param, const float* grad, float* momentum_buf, size_t n, double lr, double momentum,
+                    double dampening, double weight_decay, int nesterov, int first_step);
+/* One Adam (_functional.py:25-65) or AdamW (decoupled_weight_decay != 0, :68-119) update in place;
+ * `step` counts from 1; max_exp_avg_sq only with amsgrad.  The moments are float32 with separate
+ * roundings; the denominator sqrt(v) / sqrt(1 - beta2^step) + eps and the final update are
+ * float64, as the reference's mixed float32-array / float64-scalar expressions evaluate. */
+int tt_adam_step_f32(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, float* max_exp_avg_sq,
+                     size_t n, int step, double lr, double beta1, double beta2, double eps, double weight_decay,
+                     int amsgrad, int decoupled_weight_decay);
+
 /* ---- elementwise glue so whole stacks stay on the device ----------------------------------- */
 
 /* y = max(x, 0) (autograd/grad_nn.py:33-69); dx = dy * (y > 0). */

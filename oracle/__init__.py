@@ -26,6 +26,8 @@ publishes no golden vectors for this path):
 * ``mean_*``, ``mm_*``, ``linear_*``, ``log_softmax_*``, ``nll_loss_*``
                         torch CPU functions with autograd (weights, ignore_index, reductions),
                         closed forms (normalisation, zero-sum gradient rows, g / count)
+* ``optim.sgd``, ``optim.adam``
+                        torch CPU optimisers over several steps, closed forms
 
 The checks live in ``tests/test_oracle_*.py``.
 """
@@ -37,6 +39,7 @@ from .nninit import conv_parameters, bn_affine_c4
 from .pool import max_pool2d, max_pool2d_backward, pool_output_size
 from .head import (mean_forward, mean_backward, mm_forward, mm_backward, linear_forward, linear_backward,
                    log_softmax_forward, log_softmax_backward, nll_loss_forward, nll_loss_backward)
+from . import optim
 from .activation import relu_forward, relu_backward, leaky_relu_forward, leaky_relu_backward
 
 __all__ = [
@@ -45,6 +48,7 @@ __all__ = [
     'transposed_convolution_forward', 'transposed_convolution_backward',
     'batch_norm_forward', 'batch_norm_backward', 'conv_parameters', 'bn_affine_c4',
     'max_pool2d', 'max_pool2d_backward', 'pool_output_size',
+    'optim',
     'relu_forward', 'relu_backward', 'leaky_relu_forward', 'leaky_relu_backward',
     'mean_forward', 'mean_backward', 'mm_forward', 'mm_backward', 'linear_forward', 'linear_backward',
     'log_softmax_forward', 'log_softmax_backward', 'nll_loss_forward', 'nll_loss_backward',

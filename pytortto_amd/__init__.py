@@ -18,6 +18,7 @@ from .autograd import (no_grad, enable_grad, set_grad_enabled, is_grad_enabled, 
                        ToCopy, Add, Convolution, TransposedConvolution, BatchNorm, Relu, LeakyRelu,
                        MaxPool2DWithIndices, LogSoftmax, NllLoss, View, Transpose, Mm, Mean)
 from . import nn
+from . import optim
 from . import _hip
 
 cparray = hiparray   # the reference's name for "the device array class"

@@ -161,3 +161,28 @@ def test_cpu_copy_is_a_no_op_on_host_and_numpy_rules():
     x.requires_grad_(True)
     with pytest.raises(RuntimeError, match="Can't call numpy\\(\\) on Tensor that requires grad"):
         x.numpy()
+
+
+def test_optimizer_plumbing_on_host():
+    """Parameter groups, defaults, validation and state_dict layout need no GPU."""
+    import pytortto_amd as tt
+    lin = tt.nn.Linear(4, 2)
+    opt = tt.optim.SGD([{'params': [lin.weight]}, {'params': [lin.bias], 'lr': 0.5}], lr=0.1, momentum=0.9)
+    assert [g['lr'] for g in opt.param_groups] == [0.1, 0.5] and opt.param_groups[1]['momentum'] == 0.9
+    sd = opt.state_dict()
+    assert sd['param_groups'][0]['params'] == [0] and sd['param_groups'][1]['params'] == [1]
+    opt.load_state_dict(sd)
+    with pytest.raises(ValueError, match='Nesterov momentum requires a momentum and zero dampening'):
+        tt.optim.SGD(lin.parameters(), lr=0.1, nesterov=True)
+    with pytest.raises(ValueError, match='Invalid beta parameter at index 0'):
+        tt.optim.Adam(lin.parameters(), betas=(1.0, 0.9))
+    with pytest.raises(ValueError, match='empty parameter list'):
+        tt.optim.Adam([])
+    with pytest.raises(TypeError, match='iterable of Tensors or dicts'):
+        tt.optim.SGD(lin.weight, lr=0.1)
+    with pytest.raises(ValueError, match='more than one parameter group'):
+        tt.optim.SGD([{'params': [lin.weight]}, {'params': [lin.weight]}], lr=0.1)
+    with pytest.raises(ValueError, match="can't optimize a non-leaf Tensor"):
+        tt.optim.SGD([lin.weight + lin.weight], lr=0.1)
+    assert tt.optim.AdamW(lin.parameters()).defaults['weight_decay'] == 1e-2
+    assert 'lr: 0.1' in repr(opt)
