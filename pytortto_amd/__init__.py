@@ -17,6 +17,7 @@ from .VariableFunctions import (manual_seed, empty, zeros, ones, randn, tensor, 
 from .autograd import (no_grad, enable_grad, set_grad_enabled, is_grad_enabled, Function, AccumulateGrad,
                        ToCopy, Add, Convolution, TransposedConvolution, BatchNorm, Relu, LeakyRelu,
                        MaxPool2DWithIndices, LogSoftmax, NllLoss, View, Transpose, Mm, Mean)
+from .serialization import save, load
 from . import nn
 from . import optim
 from . import _hip

@@ -181,9 +181,10 @@ class hiparray:
 
     def set(self, host):
         """Overwrite the contents from a host array of the same shape (used by ``copy_``)."""
-        host = np.ascontiguousarray(np.asarray(host, dtype=self._dtype))
+        host = np.asarray(host, dtype=self._dtype)
         if host.shape != self._shape:
-            host = np.ascontiguousarray(np.broadcast_to(host, self._shape))
+            host = np.broadcast_to(host, self._shape)
+        host = np.ascontiguousarray(host)               # (a 0-d array comes back 1-d: same bytes)
         if host.nbytes:
             _hip.call('tt_memcpy_h2d', self.ptr, host.ctypes.data, host.nbytes)
         return self

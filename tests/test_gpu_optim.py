@@ -110,3 +110,42 @@ def test_optimizer_refuses_host_parameters():
     lin.bias.grad = np.zeros(2, np.float32)
     with pytest.raises(RuntimeError, match='device parameters only'):
         tt.optim.SGD(lin.parameters(), lr=0.1).step()
+
+
+def test_checkpoint_of_device_model_and_optimizer(tmp_path):
+    """state_dict() of device modules and of the optimiser holds host arrays; tt.save / tt.load
+    carry them, and a fresh device model resumes with identical parameters, BatchNorm buffers
+    and momentum."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    tt.manual_seed(4)
+
+    def make():
+        net = nn.Sequential(nn.Conv2d(3, 4, 3, padding=1, bias=False), nn.BatchNorm2d(4), nn.ReLU())
+        net.cuda()
+        return net, tt.optim.SGD(net.parameters(), lr=0.1, momentum=0.9)
+
+    net, opt = make()
+    x = tt.randn(8, 3, 6, 6).cuda()
+    g = tt.randn(8, 4, 6, 6).cuda()
+    for _ in range(2):
+        opt.zero_grad()
+        net(x).backward(g)
+        opt.step()
+    path = str(tmp_path / 'ckpt.npy')
+    tt.save({'model': net.state_dict(), 'optim': opt.state_dict()}, path)
+    ck = tt.load(path)
+    assert all(type(v) is np.ndarray for v in ck['model'].values())
+    assert ck['model']['1.num_batches_tracked'] == 2 and not np.allclose(ck['model']['1.running_mean'], 0)
+    net2, opt2 = make()
+    net2.load_state_dict(ck['model'])
+    opt2.load_state_dict(ck['optim'])
+    for (k, a), (_, b) in zip(net.state_dict().items(), net2.state_dict().items()):
+        np.testing.assert_array_equal(a, b, err_msg=k)
+    # one more identical step on both: same result, so the momentum buffers came along
+    for n_, o_ in ((net, opt), (net2, opt2)):
+        o_.zero_grad()
+        n_(x).backward(g)
+        o_.step()
+    for (k, a), (_, b) in zip(net.state_dict().items(), net2.state_dict().items()):
+        np.testing.assert_array_equal(a, b, err_msg=k)

@@ -186,3 +186,27 @@ def test_optimizer_plumbing_on_host():
         tt.optim.SGD([lin.weight + lin.weight], lr=0.1)
     assert tt.optim.AdamW(lin.parameters()).defaults['weight_decay'] == 1e-2
     assert 'lr: 0.1' in repr(opt)
+
+
+def test_checkpoint_wire_format_round_trip(tmp_path):
+    """tt.save writes {'data': obj} as one pickled object in a .npy file; a model's state_dict
+    (parameters and BatchNorm buffers, host arrays) survives the round trip."""
+    tt.manual_seed(5)
+    net = nn.Sequential(nn.Conv2d(3, 4, 3, bias=True), nn.BatchNorm2d(4), nn.ReLU())
+    net[1].running_mean.data[...] = np.arange(4, dtype=np.float32)
+    sd = net.state_dict()
+    assert list(sd) == ['0.weight', '0.bias', '1.weight', '1.bias', '1.running_mean', '1.running_var',
+                        '1.num_batches_tracked']
+    path = str(tmp_path / 'ckpt.npy')
+    tt.save({'model': sd, 'epoch': 3}, path)
+    raw = np.load(path, allow_pickle=True)
+    assert raw.dtype == object and raw.shape == () and set(raw.item()) == {'data'}
+    back = tt.load(path)
+    assert back['epoch'] == 3
+    other = nn.Sequential(nn.Conv2d(3, 4, 3, bias=True), nn.BatchNorm2d(4), nn.ReLU())
+    other.load_state_dict(back['model'])
+    for k, v in other.state_dict().items():
+        assert type(v) is np.ndarray
+        np.testing.assert_array_equal(v, sd[k])
+    with pytest.raises(RuntimeError, match='Missing key'):
+        other.load_state_dict({k: v for k, v in sd.items() if k != '1.running_var'})
