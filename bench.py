@@ -130,6 +130,82 @@ def profiled_steps(hip, step, steps):
     return prof
 
 
+def resnet50_train_step(hip, steps, warmup, batch=BATCH):
+    """Whole ResNet-50 training steps through the module API (the network of the reference's
+    examples/resnet/resnet50_finetune notebook, 10 classes): forward, NLL loss, backward, SGD with
+    momentum, everything on the device.  Returns (images/s, ms per step from HIP events, wall ms)."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    F = nn.functional
+
+    def conv3x3(cin, cout, stride=1):
+        return nn.Conv2d(cin, cout, kernel_size=3, stride=stride, padding=1, bias=False)
+
+    def conv1x1(cin, cout, stride=1):
+        return nn.Conv2d(cin, cout, kernel_size=1, stride=stride, bias=False)
+
+    class Bottleneck(nn.Module):
+        def __init__(self, cin, width, stride=1, downsample=None):
+            super().__init__()
+            self.conv1, self.bn1 = conv1x1(cin, width), nn.BatchNorm2d(width)
+            self.conv2, self.bn2 = conv3x3(width, width, stride), nn.BatchNorm2d(width)
+            self.conv3, self.bn3 = conv1x1(width, width * 4), nn.BatchNorm2d(width * 4)
+            self.downsample = downsample
+
+        def forward(self, x):
+            shortcut = x if self.downsample is None else self.downsample(x)
+            out = F.relu(self.bn1(self.conv1(x)))
+            out = F.relu(self.bn2(self.conv2(out)))
+            out = self.bn3(self.conv3(out))
+            return F.relu(out + shortcut)
+
+    class ResNet50(nn.Module):
+        def __init__(self, classes=10):
+            super().__init__()
+            self.conv1 = nn.Conv2d(3, 64, kernel_size=7, stride=2, padding=3, bias=False)
+            self.bn1 = nn.BatchNorm2d(64)
+            self.maxpool = nn.MaxPool2d(kernel_size=3, stride=2, padding=1)
+            blocks, cin = [], 64
+            for width, count, stride in ((64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)):
+                for i in range(count):
+                    down = None
+                    if i == 0:
+                        down = nn.Sequential(conv1x1(cin, width * 4, stride), nn.BatchNorm2d(width * 4))
+                    blocks.append(Bottleneck(cin, width, stride if i == 0 else 1, down))
+                    cin = width * 4
+            self.layers = nn.Sequential(*blocks)
+            self.classifier = nn.Linear(2048, classes)
+
+        def forward(self, x):
+            x = self.maxpool(F.relu(self.bn1(self.conv1(x))))
+            x = self.layers(x)
+            x = tt.flatten(tt.mean(x, (-1, -2), True), 1)
+            return F.log_softmax(self.classifier(x), -1)
+
+    tt.manual_seed(0)
+    net = ResNet50()
+    net.cuda()
+    opt = tt.optim.SGD(net.parameters(), lr=0.001, momentum=0.9)
+    rng = np.random.default_rng(0)
+    x = tt.tensor(rng.standard_normal((batch, 3, 224, 224), dtype=np.float32)).cuda()
+    target = tt.tensor(rng.integers(0, 10, batch)).cuda()
+    losses = []
+
+    def step():
+        opt.zero_grad()
+        loss = F.nll_loss(net(x), target)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(warmup):
+        losses.append(step().item())
+    ms, wall = timed_steps(hip, step, steps, 0)
+    losses.append(step().item())
+    del net, opt, x
+    return batch / (wall * 1e-3), ms, wall, losses
+
+
 def cpu_baseline_pool(batch):
     """(bytes counted, seconds) of the oracle's MaxPool2d forward + backward."""
     import oracle
@@ -198,6 +274,7 @@ def main():
     ap.add_argument('--steps', type=int, default=10)
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the host-side oracle timing')
+    ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this path runs on exactly one GPU (asked for --gpus {args.gpus}); '
@@ -297,6 +374,17 @@ def main():
     del px, py, ptap, pdx
     call('tt_empty_cache')
 
+    # ---- the whole network through the module API ---------------------------------------------
+    model = None
+    if not args.no_model_step:
+        ips, m_ms, m_wall, m_losses = resnet50_train_step(_hip, max(3, args.steps // 2), 2)
+        model = {'metric': 'ResNet-50 training step images/s (module API: forward, NLL loss, backward, SGD momentum)',
+                 'value': round(ips, 1), 'unit': 'images/s', 'ms_per_step': round(m_wall, 2),
+                 'gpu_ms_per_step': round(m_ms, 2), 'batch': BATCH,
+                 'loss_first_last': [round(m_losses[0], 4), round(m_losses[-1], 4)],
+                 'note': 'wall clock around the Python loop, launches asynchronous; fp32, synthetic 3x224x224 input'}
+        call('tt_empty_cache')
+
     # ---- what the device sustains on the two bounding resources, measured in this run ----------
     mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
     hbm_read, hbm_copy = _hip.probe_hbm(2 << 30)
@@ -366,6 +454,7 @@ def main():
                                             'maxpool_bwd': round(ms_pb / max(1, n_pb), 4)},
                     'elementwise_gbs_at_same_size': act,
                     'cpu_baseline': cpu_pool},
+        'resnet50_step': model,
     }
     print(json.dumps(out))
 
