@@ -221,6 +221,9 @@ int tt_add_f32(const float* a, const float* b, float* out, size_t n);
 /* acc += alpha * v: gradient accumulation `fn.grad[ind] += grad` (tensor.py:596-599,
  * autograd/function.py:88-93). */
 int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n);
+/* acc[i] += value (a Python scalar added in place, e.g. `num_batches_tracked.data += 1`,
+ * nn/modules/batchnorm.py:66). */
+int tt_add_scalar_f32(float* acc, float value, size_t n);
 /* dst[i] = value */
 int tt_fill_f32(float* dst, float value, size_t n);
 

@@ -6,7 +6,7 @@ namespace {
 
 constexpr int kThreads = 256;
 
-enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill, kLeakyRelu, kLeakyReluBwd };
+enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill, kLeakyRelu, kLeakyReluBwd, kAddScalar };
 
 template <int OP>
 __device__ __forceinline__ float apply1(float a, float b, float alpha) {
@@ -20,6 +20,7 @@ __device__ __forceinline__ float apply1(float a, float b, float alpha) {
   if (OP == kReluBwd) return b > 0.f ? a : 0.f;  // a = dy, b = y
   if (OP == kAdd) return a + b;
   if (OP == kAxpy) return fmaf(alpha, a, b);      // a = v, b = acc
+  if (OP == kAddScalar) return a + alpha;
   return alpha;                                    // kFill
 }
 
@@ -75,6 +76,9 @@ int tt_leaky_relu_bwd_f32(const float* dy, const float* x, float* dx, float nega
 int tt_add_f32(const float* a, const float* b, float* out, size_t n) { return run<kAdd>("tt_add_f32", a, b, out, 0.f, n); }
 int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n) {
   return run<kAxpy>("tt_axpy_f32", v, acc, acc, alpha, n);
+}
+int tt_add_scalar_f32(float* acc, float value, size_t n) {
+  return run<kAddScalar>("tt_add_scalar_f32", acc, nullptr, acc, value, n);
 }
 int tt_fill_f32(float* dst, float value, size_t n) { return run<kFill>("tt_fill_f32", nullptr, nullptr, dst, value, n); }
 

@@ -1,4 +1,5 @@
-"""``ReLU``, ``LeakyReLU`` and ``LogSoftmax`` (``src/tortto/nn/modules/activation.py:24-48``, ``:75-84``)."""
+"""``ReLU``, ``LeakyReLU`` and ``LogSoftmax`` (``src/tortto/nn/modules/activation.py:24-48``,
+``:75-84``): each keeps its hyper-parameters and calls the functional of the same name."""
 from .. import functional as F
 from .module import Module
 
@@ -18,15 +19,13 @@ class ReLU(Module):
 class LeakyReLU(Module):
     def __init__(self, negative_slope=1e-2, inplace=False):
         super().__init__()
-        self.negative_slope = negative_slope
-        self.inplace = inplace
+        self.negative_slope, self.inplace = negative_slope, inplace
 
     def forward(self, tensor):
         return F.leaky_relu(tensor, self.negative_slope, self.inplace)
 
     def extra_repr(self):
-        inplace_str = ', inplace=True' if self.inplace else ''
-        return f'negative_slope={self.negative_slope}{inplace_str}'
+        return f'negative_slope={self.negative_slope}' + (', inplace=True' if self.inplace else '')
 
 
 class LogSoftmax(Module):

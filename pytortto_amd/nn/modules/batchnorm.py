@@ -1,6 +1,7 @@
-"""``BatchNorm2d`` (and the 1d/3d input checks) as in ``src/tortto/nn/modules/batchnorm.py``:
-gamma=1, beta=0, running_mean=0, running_var=1, ``num_batches_tracked`` a float32 scalar tensor;
-``momentum=None`` switches to a cumulative moving average."""
+"""``BatchNorm1d/2d/3d`` modules with the state and behaviour of
+``src/tortto/nn/modules/batchnorm.py`` (:8-57 state, :62-93 forward, :104-107 and siblings for the
+input checks): gamma = 1, beta = 0, running_mean = 0, running_var = 1, ``num_batches_tracked`` a
+float32 scalar buffer; ``momentum=None`` turns the running statistics into a cumulative average."""
 from ... import VariableFunctions as _vf
 from ...tensor import Tensor
 from .. import functional as F
@@ -9,28 +10,22 @@ from ..parameter import Parameter
 from .module import Module
 
 
-class _NormBase(Module):
+class _BatchNorm(Module):
+    _input_dims = ()        # admissible input ranks, set by the subclasses
+
     def __init__(self, num_features, eps=1e-5, momentum=0.1, affine=True, track_running_stats=True):
         super().__init__()
-        self.num_features = num_features
-        self.eps = eps
-        self.momentum = momentum
-        self.affine = affine
-        self.track_running_stats = track_running_stats
-        if self.affine:
-            self.weight = Parameter(_vf.ones(num_features))
-            self.bias = Parameter(_vf.zeros(num_features))
-        else:
-            self.register_parameter('weight', None)
-            self.register_parameter('bias', None)
-        if self.track_running_stats:
+        self.__dict__.update(num_features=num_features, eps=eps, momentum=momentum, affine=affine,
+                             track_running_stats=track_running_stats)
+        for name, start in (('weight', _vf.ones), ('bias', _vf.zeros)):
+            self.register_parameter(name, Parameter(start(num_features)) if affine else None)
+        if track_running_stats:
             self.register_buffer('running_mean', _vf.zeros(num_features))
             self.register_buffer('running_var', _vf.ones(num_features))
             self.register_buffer('num_batches_tracked', Tensor(0))
         else:
-            self.register_parameter('running_mean', None)
-            self.register_parameter('running_var', None)
-            self.register_parameter('num_batches_tracked', None)
+            for name in ('running_mean', 'running_var', 'num_batches_tracked'):
+                self.register_parameter(name, None)
         self.reset_parameters()
 
     def reset_running_stats(self):
@@ -46,44 +41,36 @@ class _NormBase(Module):
             init.zeros_(self.bias)
 
     def _check_input_dim(self, input):
-        raise NotImplementedError
+        if input.dim() not in self._input_dims:
+            wanted = ' or '.join(f'{d}D' for d in self._input_dims)
+            raise ValueError(f'expected {wanted} input (got {input.dim()}D input)')
 
     def extra_repr(self):
-        return ('{num_features}, eps={eps}, momentum={momentum}, affine={affine}, '
-                'track_running_stats={track_running_stats}'.format(**self.__dict__))
+        return (f'{self.num_features}, eps={self.eps}, momentum={self.momentum}, affine={self.affine}, '
+                f'track_running_stats={self.track_running_stats}')
 
-
-class _BatchNorm(_NormBase):
     def forward(self, inpt):
         self._check_input_dim(inpt)
+        factor = None                                   # weight of the new batch in the running statistics
         if self.training and self.track_running_stats:
-            self.num_batches_tracked.data += 1
-            if self.momentum is None:
-                factor = 1.0 / self.num_batches_tracked.item()
-            else:
-                factor = self.momentum
-        else:
-            factor = None
-        bn_training = True if self.training else (self.running_mean is None and self.running_var is None)
-        use_buffers = not self.training or self.track_running_stats
-        return F.batch_norm(inpt, self.running_mean if use_buffers else None,
-                            self.running_var if use_buffers else None,
-                            self.weight, self.bias, bn_training, factor, self.eps)
+            self.num_batches_tracked.data += 1          # (:66)
+            factor = self.momentum if self.momentum is not None else 1.0 / self.num_batches_tracked.item()
+        # batch statistics are used in training mode, and in eval mode when there are no buffers (:75-78)
+        no_buffers = self.running_mean is None and self.running_var is None
+        batch_stats = self.training or no_buffers
+        pass_buffers = self.track_running_stats or not self.training
+        return F.batch_norm(inpt, self.running_mean if pass_buffers else None,
+                            self.running_var if pass_buffers else None, self.weight, self.bias, batch_stats,
+                            factor, self.eps)
 
 
 class BatchNorm1d(_BatchNorm):
-    def _check_input_dim(self, input):
-        if input.dim() != 2 and input.dim() != 3:
-            raise ValueError('expected 2D or 3D input (got {}D input)'.format(input.dim()))
+    _input_dims = (2, 3)
 
 
 class BatchNorm2d(_BatchNorm):
-    def _check_input_dim(self, input):
-        if input.dim() != 4:
-            raise ValueError('expected 4D input (got {}D input)'.format(input.dim()))
+    _input_dims = (4,)
 
 
 class BatchNorm3d(_BatchNorm):
-    def _check_input_dim(self, input):
-        if input.dim() != 5:
-            raise ValueError('expected 5D input (got {}D input)'.format(input.dim()))
+    _input_dims = (5,)

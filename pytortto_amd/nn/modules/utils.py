@@ -1,14 +1,11 @@
-from collections.abc import Iterable
-from itertools import repeat
+"""Argument helpers of the modules (``src/tortto/nn/modules/utils.py``)."""
 
 
 def _ntuple(n):
+    """int -> n-tuple of it; a sequence -> its first n entries."""
     def parse(x):
-        if isinstance(x, Iterable):
-            return x[:n]
-        return tuple(repeat(x, n))
+        return tuple(x[:n]) if hasattr(x, '__iter__') else (x,) * n
     return parse
 
 
-_single = _ntuple(1)
-_pair = _ntuple(2)
+_single, _pair = _ntuple(1), _ntuple(2)

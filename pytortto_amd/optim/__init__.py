@@ -1,6 +1,5 @@
 """``tt.optim``: the optimisers that consume the gradients of the path (``src/tortto/optim``)."""
 from .optimizer import Optimizer
-from .adam import Adam, AdamW
-from .sgd import SGD
+from .rules import SGD, Adam, AdamW
 
 __all__ = ['Optimizer', 'SGD', 'Adam', 'AdamW']

@@ -1,10 +1,9 @@
-"""``Optimizer`` base class (``src/tortto/optim/optimizer.py``): parameter groups, per-parameter
-state, ``zero_grad``, ``state_dict`` / ``load_state_dict`` (state arrays are saved as NumPy
-arrays and moved to the parameter's device on load, :68-79, :108-123)."""
-import collections.abc
+"""``Optimizer``: parameter groups with per-group hyper-parameters, per-parameter state,
+``zero_grad`` and the ``state_dict`` layout of ``src/tortto/optim/optimizer.py`` (groups refer to
+parameters by running index; state arrays are saved as host NumPy arrays, :68-79, and moved to
+each parameter's device when loaded, :108-123)."""
 import warnings
 from collections import defaultdict
-from itertools import chain
 
 import numpy as np
 
@@ -13,6 +12,8 @@ from ..xparray import hiparray
 
 
 class _RequiredParameter:
+    """Marks a hyper-parameter that every group has to supply (``lr`` of SGD)."""
+
     def __repr__(self):
         return '<required parameter>'
 
@@ -20,86 +21,67 @@ class _RequiredParameter:
 required = _RequiredParameter()
 
 
+def _to_host(value):
+    return value.get() if value.__class__ is hiparray else value
+
+
+def _like(param, value):
+    """``value`` of a loaded checkpoint, with arrays placed where ``param`` lives."""
+    if isinstance(value, np.ndarray):
+        return hiparray(value) if param.data.__class__ is hiparray else value
+    if isinstance(value, dict):
+        return {k: _like(param, v) for k, v in value.items()}
+    if isinstance(value, (list, tuple)):
+        return type(value)(_like(param, v) for v in value)
+    return value
+
+
 class Optimizer:
     def __init__(self, params, defaults):
-        self.defaults = defaults
         if isinstance(params, Tensor):
             raise TypeError('params argument given to the optimizer should be an iterable of Tensors or dicts, '
                             'but got ' + params.__class__.__name__)
+        self.defaults = defaults
         self.state = defaultdict(dict)
         self.param_groups = []
-        param_groups = list(params)
-        if len(param_groups) == 0:
+        groups = list(params)
+        if not groups:
             raise ValueError('optimizer got an empty parameter list')
-        if not isinstance(param_groups[0], dict):
-            param_groups = [{'params': param_groups}]
-        for group in param_groups:
+        if not isinstance(groups[0], dict):
+            groups = [{'params': groups}]
+        for group in groups:
             self.add_param_group(group)
 
-    def __getstate__(self):
-        return {'defaults': self.defaults, 'state': self.state, 'param_groups': self.param_groups}
+    # ---- groups -------------------------------------------------------------------------------------
+    def add_param_group(self, param_group):
+        assert isinstance(param_group, dict), 'param group must be a dict'
+        members = param_group['params']
+        if isinstance(members, set):
+            raise TypeError('optimizer parameters need to be organized in ordered collections, but the ordering of '
+                            'tensors in sets will change between runs. Please use a list instead.')
+        members = [members] if isinstance(members, Tensor) else list(members)
+        for p in members:
+            if not isinstance(p, Tensor):
+                raise TypeError('optimizer can only optimize Tensors, but one of the params is ' +
+                                p.__class__.__name__)
+            if not p.is_leaf:
+                raise ValueError("can't optimize a non-leaf Tensor")
+        param_group['params'] = members
+        for name, default in self.defaults.items():
+            if default is required and name not in param_group:
+                raise ValueError("parameter group didn't specify a value of required optimization parameter " + name)
+            param_group.setdefault(name, default)
+        if len(set(members)) != len(members):
+            warnings.warn('optimizer contains a parameter group with duplicate parameters.', stacklevel=3)
+        taken = {p for group in self.param_groups for p in group['params']}
+        if taken & set(members):
+            raise ValueError('some parameters appear in more than one parameter group')
+        self.param_groups.append(param_group)
 
-    def __setstate__(self, state):
-        self.__dict__.update(state)
-
-    def __repr__(self):
-        text = self.__class__.__name__ + ' ('
-        for i, group in enumerate(self.param_groups):
-            text += f'\nParameter Group {i}\n'
-            for key in sorted(group.keys()):
-                if key != 'params':
-                    text += f'    {key}: {group[key]}\n'
-        return text + ')'
-
-    def state_dict(self):
-        index_of = {}
-        start = 0
-        packed_groups = []
+    def _with_grad(self):
+        """(group, parameters of the group that received a gradient) for every group."""
         for group in self.param_groups:
-            packed = {k: v for k, v in group.items() if k != 'params'}
-            index_of.update({id(p): i for i, p in enumerate(group['params'], start) if id(p) not in index_of})
-            packed['params'] = [index_of[id(p)] for p in group['params']]
-            start += len(packed['params'])
-            packed_groups.append(packed)
-
-        def to_host(entry):
-            return {k: v.get() if v.__class__ is hiparray else v for k, v in entry.items()}
-
-        packed_state = {(index_of[id(k)] if isinstance(k, Tensor) else k): to_host(v) for k, v in self.state.items()}
-        return {'state': packed_state, 'param_groups': packed_groups}
-
-    def load_state_dict(self, state_dict):
-        state_dict = state_dict.copy()
-        groups, saved_groups = self.param_groups, state_dict['param_groups']
-        if len(groups) != len(saved_groups):
-            raise ValueError('loaded state dict has a different number of parameter groups')
-        if any(len(g['params']) != len(s['params']) for g, s in zip(groups, saved_groups)):
-            raise ValueError("loaded state dict contains a parameter group that doesn't match the size of "
-                             "optimizer's group")
-        by_index = dict(zip(chain.from_iterable(g['params'] for g in saved_groups),
-                            chain.from_iterable(g['params'] for g in groups)))
-
-        def cast(param, value):
-            if isinstance(value, np.ndarray):
-                return hiparray(value) if param.data.__class__ is hiparray else value
-            if isinstance(value, dict):
-                return {k: cast(param, v) for k, v in value.items()}
-            if isinstance(value, collections.abc.Iterable) and not isinstance(value, str):
-                return type(value)(cast(param, v) for v in value)
-            return value
-
-        state = defaultdict(dict)
-        for k, v in state_dict['state'].items():
-            if k in by_index:
-                state[by_index[k]] = cast(by_index[k], v)
-            else:
-                state[k] = v
-        new_groups = []
-        for group, saved in zip(groups, saved_groups):
-            saved = dict(saved)
-            saved['params'] = group['params']
-            new_groups.append(saved)
-        self.__setstate__({'state': state, 'param_groups': new_groups})
+            yield group, [p for p in group['params'] if p.grad is not None and p.grad.__class__ is not int]
 
     def zero_grad(self):
         for group in self.param_groups:
@@ -109,32 +91,46 @@ class Optimizer:
     def step(self):
         raise NotImplementedError
 
-    def add_param_group(self, param_group):
-        assert isinstance(param_group, dict), 'param group must be a dict'
-        params = param_group['params']
-        if isinstance(params, Tensor):
-            param_group['params'] = [params]
-        elif isinstance(params, set):
-            raise TypeError('optimizer parameters need to be organized in ordered collections, but the ordering of '
-                            'tensors in sets will change between runs. Please use a list instead.')
-        else:
-            param_group['params'] = list(params)
-        for param in param_group['params']:
-            if not isinstance(param, Tensor):
-                raise TypeError('optimizer can only optimize Tensors, but one of the params is ' +
-                                param.__class__.__name__)
-            if not param.is_leaf:
-                raise ValueError("can't optimize a non-leaf Tensor")
-        for name, default in self.defaults.items():
-            if default is required and name not in param_group:
-                raise ValueError("parameter group didn't specify a value of required optimization parameter " + name)
-            param_group.setdefault(name, default)
-        params = param_group['params']
-        if len(params) != len(set(params)):
-            warnings.warn('optimizer contains a parameter group with duplicate parameters.', stacklevel=3)
-        seen = set()
+    # ---- (de)serialisation ---------------------------------------------------------------------------
+    def __getstate__(self):
+        return {'defaults': self.defaults, 'state': self.state, 'param_groups': self.param_groups}
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+
+    def state_dict(self):
+        number = {}
         for group in self.param_groups:
-            seen.update(group['params'])
-        if not seen.isdisjoint(param_group['params']):
-            raise ValueError('some parameters appear in more than one parameter group')
-        self.param_groups.append(param_group)
+            for p in group['params']:
+                number.setdefault(id(p), len(number))
+        groups = [{**{k: v for k, v in g.items() if k != 'params'}, 'params': [number[id(p)] for p in g['params']]}
+                  for g in self.param_groups]
+        state = {(number[id(k)] if isinstance(k, Tensor) else k): {name: _to_host(v) for name, v in entry.items()}
+                 for k, entry in self.state.items()}
+        return {'state': state, 'param_groups': groups}
+
+    def load_state_dict(self, state_dict):
+        saved_groups = state_dict['param_groups']
+        if len(saved_groups) != len(self.param_groups):
+            raise ValueError('loaded state dict has a different number of parameter groups')
+        for mine, saved in zip(self.param_groups, saved_groups):
+            if len(mine['params']) != len(saved['params']):
+                raise ValueError("loaded state dict contains a parameter group that doesn't match the size of "
+                                 "optimizer's group")
+        owner = {index: p for mine, saved in zip(self.param_groups, saved_groups)
+                 for index, p in zip(saved['params'], mine['params'])}
+        state = defaultdict(dict)
+        for key, entry in state_dict['state'].items():
+            if key in owner:
+                state[owner[key]] = _like(owner[key], entry)
+            else:
+                state[key] = entry
+        groups = [{**saved, 'params': mine['params']} for mine, saved in zip(self.param_groups, saved_groups)]
+        self.__setstate__({'state': state, 'param_groups': groups})
+
+    def __repr__(self):
+        lines = [self.__class__.__name__ + ' (']
+        for i, group in enumerate(self.param_groups):
+            lines.append(f'Parameter Group {i}')
+            lines += [f'    {key}: {group[key]}' for key in sorted(group) if key != 'params']
+        return '\n'.join(lines) + '\n)'

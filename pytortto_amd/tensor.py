@@ -227,3 +227,18 @@ class Tensor:
             acc.variable = self
             acc.grad = (gradient,)
             acc.apply(*acc.grad)
+
+
+class Parameter(Tensor):
+    """``nn.Parameter`` (``src/tortto/nn/parameter.py``): a leaf tensor that asks for a gradient by
+    default and adopts -- does not copy -- the array of the tensor it is made from."""
+
+    def __init__(self, data=None, requires_grad=True, **kwargs):
+        if data is not None and not isinstance(data, Tensor):
+            raise TypeError(f'input must be Tensor, not {data.__class__.__name__}')
+        array = None if data is None else data.data
+        super().__init__(array, requires_grad=requires_grad, dtype=float32 if array is None else array.dtype,
+                         copy=False)
+
+    def __repr__(self):
+        return 'Parameter containing:\n' + super().__repr__()

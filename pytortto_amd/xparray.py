@@ -223,10 +223,8 @@ class hiparray:
             if self.size:
                 _hip.call('tt_axpy_f32', 1.0, other.ptr, self.ptr, self.size)
         elif isinstance(other, (int, float, np.floating, np.integer)):
-            tmp = hiparray.empty(self._shape, self._dtype)
-            tmp.fill(other)
             if self.size:
-                _hip.call('tt_axpy_f32', 1.0, tmp.ptr, self.ptr, self.size)
+                _hip.call('tt_add_scalar_f32', self.ptr, float(other), self.size)
         else:
             raise TypeError(f'device += is not defined for {other.__class__.__name__}')
         return self
