@@ -49,6 +49,7 @@ BATCH = 64
 # (bench_hbm_traffic_fetch_write_size.txt).
 IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 237.1e6      # igemm_f32 + igemm_multi_f32 + igemm_fixup, mean over the 106 launches of a step (106.9e6 algorithmic)
 BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.3e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
+MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH = 314.6e6    # dy + taps read, dx written (308.3e6 algorithmic)
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
 
 
@@ -448,7 +449,8 @@ def main():
                                            '(ResNet-50 stem pooling); bytes: x + y + int32 taps, both ways'},
                     'roofline': {'bound': 'hbm', 'kernel': 'maxpool_bwd_scatter (reads dy, taps; writes dx)',
                                  'achieved': round(pool_bwd_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                                 'frac': round(pool_bwd_gbs / PEAK_HBM_GBS, 4), 'traffic': None,
+                                 'frac': round(pool_bwd_gbs / PEAK_HBM_GBS, 4),
+                                 'traffic': MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH,
                                  'avg_launch_ms': round(ms_pb / max(1, n_pb), 5)},
                     'kernels_ms_per_step': {'maxpool_fwd': round(ms_pf / max(1, n_pf), 4),
                                             'maxpool_bwd': round(ms_pb / max(1, n_pb), 4)},
