@@ -276,6 +276,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the host-side oracle timing')
     ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
+    ap.add_argument('--model-step-only', action='store_true',
+                    help='run only the whole-network ResNet-50 training step and print its object (for profiling)')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this path runs on exactly one GPU (asked for --gpus {args.gpus}); '
@@ -291,6 +293,14 @@ def main():
     info = _hip.device_info()
     call = _hip.call
     rng = np.random.default_rng(0)
+    if args.model_step_only:
+        ips, m_ms, m_wall, m_losses = resnet50_train_step(_hip, args.steps, args.warmup)
+        print(json.dumps({'metric': 'ResNet-50 training step images/s (module API)', 'value': round(ips, 1),
+                          'unit': 'images/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                          'ms_per_step': round(m_wall, 2), 'gpu_ms_per_step': round(m_ms, 2), 'batch': BATCH,
+                          'higher_is_better': True, 'dtype': 'f32', 'data': 'synthetic',
+                          'loss_first_last': [round(m_losses[0], 4), round(m_losses[-1], 4)]}))
+        return
 
     # ---- convolution: ResNet-50, batch 64 ------------------------------------------------------
     layers = [ConvLayer(spec, BATCH, rng) for spec in RESNET50_CONVS]
