@@ -149,3 +149,50 @@ def test_channel_sum_matches_numpy():
         ref = t.astype(np.float64).sum((0, 2, 3))
         got = ops.channel_sum(hiparray(t)).get()
         np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5 * np.abs(ref).max())
+
+
+@pytest.mark.parametrize('shape', [(64, 256, 56, 56), (128, 64, 112, 112)])
+def test_bn_benchmark_shapes_full_size(shape):
+    """The two shapes the BatchNorm metric is quoted on, x ~ N(2, 3): the float32 oracle for y, dx
+    and the statistics; float64 reductions for the per-channel sums; and what the algebra fixes:
+    mean(y) = beta, var(y) = gamma^2 var / (var + eps), sum(dx) = 0, sum(dx * xhat) = 0."""
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(11)
+    n, c, h, w = shape
+    x = (2 + 3 * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    gamma = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(c)).astype(np.float32)
+    rm0, rv0 = np.zeros(c, np.float32), np.ones(c, np.float32)
+    xd, dyd, gd = hiparray(x), hiparray(dy), hiparray(gamma)
+    y, mean, var_eps, sd, rm, rv = ops.bn_fwd_train(xd, gd, hiparray(beta), hiparray(rm0), hiparray(rv0), 0.1, 1e-5)
+    dx, dg, db = ops.bn_bwd(xd, dyd, gd, mean, var_eps, sd)
+    y, dx = y.get(), dx.get()
+
+    axis, m = (0, 2, 3), n * h * w
+    mu64 = x.mean(axis, dtype=np.float64)
+    var64 = ((x.astype(np.float64) - mu64[None, :, None, None]) ** 2).mean(axis)
+    np.testing.assert_allclose(mean.get(), mu64, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(var_eps.get(), var64 + 1e-5, rtol=2e-6)
+    np.testing.assert_allclose(rm.get(), 0.1 * mu64, rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(rv.get(), 0.9 + 0.1 * var64 * (m / (m - 1)), rtol=1e-5)
+
+    y_ref, saved, rm_ref, rv_ref = oracle.batch_norm_forward(x, gamma, beta, rm0, rv0, True, 0.1, 1e-5)
+    _close(y, y_ref, name='y')
+    _close(rm.get(), rm_ref, name='running_mean')
+    _close(rv.get(), rv_ref, name='running_var')
+    np.testing.assert_allclose(y.mean(axis, dtype=np.float64), beta, atol=2e-6)
+    np.testing.assert_allclose(y.var(axis, dtype=np.float64), gamma.astype(np.float64) ** 2 * var64 / (var64 + 1e-5),
+                               rtol=1e-5)
+
+    dx_ref, dg_ref, db_ref = oracle.batch_norm_backward(dy, x, gamma, saved)
+    xhat = (x.astype(np.float64) - mu64[None, :, None, None]) / np.sqrt(var64 + 1e-5)[None, :, None, None]
+    db64 = dy.sum(axis, dtype=np.float64)
+    dg64 = (dy * xhat).sum(axis)
+    np.testing.assert_allclose(db.get(), db64, rtol=1e-5, atol=1e-5 * np.abs(db64).max())
+    np.testing.assert_allclose(dg.get(), dg64, rtol=1e-5, atol=1e-5 * np.abs(dg64).max())
+    _close(dx, dx_ref, rtol=1e-4, atol_scale=1e-5, name='dx')
+    scale = float(np.abs(dx).sum(axis, dtype=np.float64).max())
+    assert np.abs(dx.sum(axis, dtype=np.float64)).max() <= 1e-5 * scale
+    assert np.abs((dx * xhat).sum(axis)).max() <= 1e-4 * scale          # exact only up to O(eps / var)
