@@ -198,6 +198,12 @@ int tt_nll_loss_bwd_f32(const float* g, const long long* target, const float* we
  * rounded to float32 separately, as NumPy evaluates the reference's expressions. */
 int tt_sgd_step_f32(float* param, const float* grad, float* momentum_buf, size_t n, double lr, double momentum,
                     double dampening, double weight_decay, int nesterov, int first_step);
+/* The same update for `count` parameters of one group (the loop of _functional.py:5) in a few
+ * launches instead of one per parameter.  The tables are host arrays; first_steps[i] != 0 marks a
+ * parameter whose momentum buffer is being created by this step. */
+int tt_sgd_step_multi_f32(int count, float* const* params, const float* const* grads, float* const* momentum_bufs,
+                          const size_t* sizes, const int* first_steps, double lr, double momentum, double dampening,
+                          double weight_decay, int nesterov);
 /* One Adam (_functional.py:25-65) or AdamW (decoupled_weight_decay != 0, :68-119) update in place;
  * `step` counts from 1; max_exp_avg_sq only with amsgrad.  The moments are float32 with separate
  * roundings; the denominator sqrt(v) / sqrt(1 - beta2^step) + eps and the final update are
@@ -205,6 +211,12 @@ int tt_sgd_step_f32(float* param, const float* grad, float* momentum_buf, size_t
 int tt_adam_step_f32(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, float* max_exp_avg_sq,
                      size_t n, int step, double lr, double beta1, double beta2, double eps, double weight_decay,
                      int amsgrad, int decoupled_weight_decay);
+/* The same for `count` parameters of one group in a few launches; steps[i] is each parameter's own
+ * step count (adam.py:60-63). */
+int tt_adam_step_multi_f32(int count, float* const* params, const float* const* grads, float* const* exp_avgs,
+                           float* const* exp_avg_sqs, float* const* max_exp_avg_sqs, const size_t* sizes,
+                           const int* steps, double lr, double beta1, double beta2, double eps, double weight_decay,
+                           int amsgrad, int decoupled_weight_decay);
 
 /* ---- elementwise glue so whole stacks stay on the device ----------------------------------- */
 

@@ -56,7 +56,9 @@ PROTOTYPES = {
     'tt_nll_loss_fwd_f32': [_P, _P, _P, _P, _P, _I, _I, ctypes.c_longlong, _I],
     'tt_nll_loss_bwd_f32': [_P, _P, _P, _P, _P, _I, _I, ctypes.c_longlong, _I],
     'tt_sgd_step_f32': [_P, _P, _P, c_size_t, c_double, c_double, c_double, c_double, _I, _I],
+    'tt_sgd_step_multi_f32': [_I, _P, _P, _P, _P, _P, c_double, c_double, c_double, c_double, _I],
     'tt_adam_step_f32': [_P, _P, _P, _P, _P, c_size_t, _I, c_double, c_double, c_double, c_double, c_double, _I, _I],
+    'tt_adam_step_multi_f32': [_I, _P, _P, _P, _P, _P, _P, _P, c_double, c_double, c_double, c_double, c_double, _I, _I],
     'tt_add_f32': [_P, _P, _P, c_size_t],
     'tt_axpy_f32': [c_float, _P, _P, c_size_t],
     'tt_add_scalar_f32': [_P, c_float, c_size_t],

@@ -29,10 +29,10 @@ struct Sgd {
   int nesterov, first, has_buf;
 };
 
-__global__ __launch_bounds__(kThreads) void sgd_step(float* __restrict__ param, const float* __restrict__ grad,
-                                                     float* __restrict__ buf, size_t n, Sgd a) {
-  const size_t stride = (size_t)gridDim.x * kThreads;
-  for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
+__device__ __forceinline__ void sgd_range(float* __restrict__ param, const float* __restrict__ grad,
+                                          float* __restrict__ buf, size_t n, size_t start, size_t stride,
+                                          const Sgd& a) {
+  for (size_t i = start; i < n; i += stride) {
     const float p = param[i];
     float d = grad[i];
     if (a.weight_decay != 0.f) d = add(d, mul(p, a.weight_decay));          // :8
@@ -51,17 +51,44 @@ __global__ __launch_bounds__(kThreads) void sgd_step(float* __restrict__ param, 
   }
 }
 
+__global__ __launch_bounds__(kThreads) void sgd_step(float* __restrict__ param, const float* __restrict__ grad,
+                                                     float* __restrict__ buf, size_t n, Sgd a) {
+  sgd_range(param, grad, buf, n, (size_t)blockIdx.x * kThreads + threadIdx.x, (size_t)gridDim.x * kThreads, a);
+}
+
+// Several parameters in one launch: blocks [first_block[t], first_block[t+1]) work on tensor t.
+// A network has one launch-bound update per parameter otherwise (161 for ResNet-50).
+constexpr int kMultiMax = 24;
+struct Tensors {
+  float* param[kMultiMax];
+  const float* grad[kMultiMax];
+  float* buf[kMultiMax];
+  unsigned long long n[kMultiMax];
+  unsigned first_block[kMultiMax + 1];
+  unsigned first_step_mask;      // bit t: tensor t takes its first momentum step
+  int count;
+};
+
+__global__ __launch_bounds__(kThreads) void sgd_step_multi(Tensors ts, Sgd a) {
+  int t = 0;
+  while (t + 1 < ts.count && blockIdx.x >= ts.first_block[t + 1]) ++t;
+  const unsigned blocks = ts.first_block[t + 1] - ts.first_block[t];
+  a.first = (ts.first_step_mask >> t) & 1;
+  sgd_range(ts.param[t], ts.grad[t], ts.buf[t], (size_t)ts.n[t],
+            (size_t)(blockIdx.x - ts.first_block[t]) * kThreads + threadIdx.x, (size_t)blocks * kThreads, a);
+}
+
 struct Adam {
   float beta1, beta2, one_minus_beta1, one_minus_beta2, weight_decay, neg_step_size, decay_factor;
   double sqrt_bias_correction2, eps;
   int amsgrad, decoupled;
 };
 
-__global__ __launch_bounds__(kThreads) void adam_step(float* __restrict__ param, const float* __restrict__ grad,
-                                                      float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
-                                                      float* __restrict__ max_exp_avg_sq, size_t n, Adam a) {
-  const size_t stride = (size_t)gridDim.x * kThreads;
-  for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
+__device__ __forceinline__ void adam_range(float* __restrict__ param, const float* __restrict__ grad,
+                                           float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
+                                           float* __restrict__ max_exp_avg_sq, size_t n, size_t start,
+                                           size_t stride, const Adam& a) {
+  for (size_t i = start; i < n; i += stride) {
     float p = param[i];
     float g = grad[i];
     if (a.decoupled) {
@@ -88,6 +115,36 @@ __global__ __launch_bounds__(kThreads) void adam_step(float* __restrict__ param,
     const double update = (double)mul(a.neg_step_size, m) / denom;                // :64
     param[i] = (float)((double)p + update);
   }
+}
+
+__global__ __launch_bounds__(kThreads) void adam_step(float* __restrict__ param, const float* __restrict__ grad,
+                                                      float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
+                                                      float* __restrict__ max_exp_avg_sq, size_t n, Adam a) {
+  adam_range(param, grad, exp_avg, exp_avg_sq, max_exp_avg_sq, n, (size_t)blockIdx.x * kThreads + threadIdx.x,
+             (size_t)gridDim.x * kThreads, a);
+}
+
+struct AdamTensors {
+  float* param[kMultiMax];
+  const float* grad[kMultiMax];
+  float* exp_avg[kMultiMax];
+  float* exp_avg_sq[kMultiMax];
+  float* max_exp_avg_sq[kMultiMax];
+  unsigned long long n[kMultiMax];
+  double sqrt_bias_correction2[kMultiMax];   // the step count, and with it the corrections, is per parameter
+  float neg_step_size[kMultiMax];
+  unsigned first_block[kMultiMax + 1];
+  int count;
+};
+
+__global__ __launch_bounds__(kThreads) void adam_step_multi(AdamTensors ts, Adam a) {
+  int t = 0;
+  while (t + 1 < ts.count && blockIdx.x >= ts.first_block[t + 1]) ++t;
+  const unsigned blocks = ts.first_block[t + 1] - ts.first_block[t];
+  a.neg_step_size = ts.neg_step_size[t];
+  a.sqrt_bias_correction2 = ts.sqrt_bias_correction2[t];
+  adam_range(ts.param[t], ts.grad[t], ts.exp_avg[t], ts.exp_avg_sq[t], ts.max_exp_avg_sq[t], (size_t)ts.n[t],
+             (size_t)(blockIdx.x - ts.first_block[t]) * kThreads + threadIdx.x, (size_t)blocks * kThreads, a);
 }
 
 unsigned blocks_for(size_t n) {
@@ -118,6 +175,51 @@ int tt_sgd_step_f32(float* param, const float* grad, float* momentum_buf, size_t
   return 0;
 }
 
+int tt_sgd_step_multi_f32(int count, float* const* params, const float* const* grads, float* const* momentum_bufs,
+                          const size_t* sizes, const int* first_steps, double lr, double momentum, double dampening,
+                          double weight_decay, int nesterov) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(count >= 0, "tt_sgd_step_multi_f32: negative count");
+  TT_REQUIRE(count == 0 || (params && grads && sizes), "tt_sgd_step_multi_f32: null table");
+  TT_REQUIRE(momentum == 0.0 || (momentum_bufs && first_steps), "tt_sgd_step_multi_f32: momentum needs buffers");
+  Sgd a;
+  a.neg_lr = (float)(-lr);
+  a.momentum = (float)momentum;
+  a.one_minus_dampening = (float)(1.0 - dampening);
+  a.weight_decay = (float)weight_decay;
+  a.nesterov = nesterov;
+  a.first = 0;
+  a.has_buf = momentum != 0.0;
+  for (int i = 0; i < count; ++i) {
+    TT_REQUIRE(sizes[i] == 0 || (params[i] && grads[i]), "tt_sgd_step_multi_f32: null pointer for tensor %d", i);
+    TT_REQUIRE(!a.has_buf || sizes[i] == 0 || momentum_bufs[i], "tt_sgd_step_multi_f32: tensor %d has no buffer", i);
+  }
+  int done = 0;
+  while (done < count) {
+    Tensors ts;
+    ts.count = 0;
+    ts.first_step_mask = 0;
+    unsigned blocks = 0;
+    for (; done < count && ts.count < kMultiMax; ++done) {
+      if (sizes[done] == 0) continue;
+      const int t = ts.count++;
+      ts.param[t] = params[done];
+      ts.grad[t] = grads[done];
+      ts.buf[t] = a.has_buf ? momentum_bufs[done] : nullptr;
+      ts.n[t] = sizes[done];
+      ts.first_block[t] = blocks;
+      if (a.has_buf && first_steps[done]) ts.first_step_mask |= 1u << t;
+      const size_t want = (sizes[done] + 4 * kThreads - 1) / (4 * kThreads);     // about four elements per thread
+      blocks += (unsigned)(want < 2048 ? want : 2048);
+    }
+    if (ts.count == 0) break;
+    ts.first_block[ts.count] = blocks;
+    sgd_step_multi<<<blocks, kThreads, 0, tt::stream()>>>(ts, a);
+    TT_LAUNCH_CHECK();
+  }
+  return 0;
+}
+
 int tt_adam_step_f32(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, float* max_exp_avg_sq,
                      size_t n, int step, double lr, double beta1, double beta2, double eps, double weight_decay,
                      int amsgrad, int decoupled_weight_decay) {
@@ -142,6 +244,61 @@ int tt_adam_step_f32(float* param, const float* grad, float* exp_avg, float* exp
   a.decoupled = decoupled_weight_decay;
   adam_step<<<blocks_for(n), kThreads, 0, tt::stream()>>>(param, grad, exp_avg, exp_avg_sq, max_exp_avg_sq, n, a);
   TT_LAUNCH_CHECK();
+  return 0;
+}
+
+int tt_adam_step_multi_f32(int count, float* const* params, const float* const* grads, float* const* exp_avgs,
+                           float* const* exp_avg_sqs, float* const* max_exp_avg_sqs, const size_t* sizes,
+                           const int* steps, double lr, double beta1, double beta2, double eps, double weight_decay,
+                           int amsgrad, int decoupled_weight_decay) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(count >= 0, "tt_adam_step_multi_f32: negative count");
+  TT_REQUIRE(count == 0 || (params && grads && exp_avgs && exp_avg_sqs && sizes && steps),
+             "tt_adam_step_multi_f32: null table");
+  TT_REQUIRE(!amsgrad || max_exp_avg_sqs, "tt_adam_step_multi_f32: amsgrad needs max_exp_avg_sq");
+  Adam a;
+  a.beta1 = (float)beta1;
+  a.beta2 = (float)beta2;
+  a.one_minus_beta1 = (float)(1.0 - beta1);
+  a.one_minus_beta2 = (float)(1.0 - beta2);
+  a.weight_decay = (float)weight_decay;
+  a.neg_step_size = 0.f;
+  a.decay_factor = (float)(1.0 - lr * weight_decay);
+  a.sqrt_bias_correction2 = 1.0;
+  a.eps = eps;
+  a.amsgrad = amsgrad;
+  a.decoupled = decoupled_weight_decay;
+  for (int i = 0; i < count; ++i) {
+    if (sizes[i] == 0) continue;
+    TT_REQUIRE(params[i] && grads[i] && exp_avgs[i] && exp_avg_sqs[i] && (!amsgrad || max_exp_avg_sqs[i]),
+               "tt_adam_step_multi_f32: null pointer for tensor %d", i);
+    TT_REQUIRE(steps[i] >= 1, "tt_adam_step_multi_f32: step counts from 1 (tensor %d)", i);
+  }
+  int done = 0;
+  while (done < count) {
+    AdamTensors ts;
+    ts.count = 0;
+    unsigned blocks = 0;
+    for (; done < count && ts.count < kMultiMax; ++done) {
+      if (sizes[done] == 0) continue;
+      const int t = ts.count++;
+      ts.param[t] = params[done];
+      ts.grad[t] = grads[done];
+      ts.exp_avg[t] = exp_avgs[done];
+      ts.exp_avg_sq[t] = exp_avg_sqs[done];
+      ts.max_exp_avg_sq[t] = amsgrad ? max_exp_avg_sqs[done] : nullptr;
+      ts.n[t] = sizes[done];
+      ts.neg_step_size[t] = (float)(-(lr / (1.0 - pow(beta1, (double)steps[done]))));
+      ts.sqrt_bias_correction2[t] = sqrt(1.0 - pow(beta2, (double)steps[done]));
+      ts.first_block[t] = blocks;
+      const size_t want = (sizes[done] + 4 * kThreads - 1) / (4 * kThreads);
+      blocks += (unsigned)(want < 2048 ? want : 2048);
+    }
+    if (ts.count == 0) break;
+    ts.first_block[ts.count] = blocks;
+    adam_step_multi<<<blocks, kThreads, 0, tt::stream()>>>(ts, a);
+    TT_LAUNCH_CHECK();
+  }
   return 0;
 }
 

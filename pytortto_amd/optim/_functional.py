@@ -1,5 +1,7 @@
-"""The update rules (``src/tortto/optim/_functional.py``) as one fused kernel launch per parameter.
+"""The update rules (``src/tortto/optim/_functional.py``) as fused kernels, a group's parameters in a few launches.
 Device parameters only: host tensors belong to tortto's NumPy path and are refused."""
+import ctypes
+
 import numpy as np
 
 from .. import _hip
@@ -14,27 +16,37 @@ def _device(param, *arrays):
 
 
 def sgd(params, d_p_list, momentum_buffer_list, weight_decay, momentum, lr, dampening, nesterov):
-    """_functional.py:4-22."""
+    """_functional.py:4-22, all parameters of the group in one call (a few launches)."""
+    count = len(params)
+    if count == 0:
+        return
+    first = [0] * count
     for i, param in enumerate(params):
-        d_p, buf = d_p_list[i], momentum_buffer_list[i]
-        _device(param, d_p, buf)
-        first = False
-        if momentum != 0 and buf is None:
-            buf = hiparray.empty(param.data.shape)      # the kernel stores d_p into it (:12-13)
-            momentum_buffer_list[i] = buf
-            first = True
-        _hip.call('tt_sgd_step_f32', param.data.ptr, d_p.ptr, None if buf is None else buf.ptr, param.data.size,
-                  lr, momentum, dampening, weight_decay, int(bool(nesterov)), int(first))
+        _device(param, d_p_list[i], momentum_buffer_list[i])
+        if momentum != 0 and momentum_buffer_list[i] is None:
+            momentum_buffer_list[i] = hiparray.empty(param.data.shape)      # the kernel stores d_p into it (:12-13)
+            first[i] = 1
+    pointers = ctypes.c_void_p * count
+    bufs = pointers(*[None if b is None else b.ptr for b in momentum_buffer_list])
+    _hip.call('tt_sgd_step_multi_f32', count, pointers(*[p.data.ptr for p in params]),
+              pointers(*[g.ptr for g in d_p_list]), bufs, (ctypes.c_size_t * count)(*[p.data.size for p in params]),
+              (ctypes.c_int * count)(*first), lr, momentum, dampening, weight_decay, int(bool(nesterov)))
 
 
 def _adam(params, grads, exp_avgs, exp_avg_sqs, max_exp_avg_sqs, state_steps, amsgrad, beta1, beta2, lr,
           weight_decay, eps, decoupled):
+    count = len(params)
+    if count == 0:
+        return
     for i, param in enumerate(params):
-        vmax = max_exp_avg_sqs[i] if amsgrad else None
-        _device(param, grads[i], exp_avgs[i], exp_avg_sqs[i], vmax)
-        _hip.call('tt_adam_step_f32', param.data.ptr, grads[i].ptr, exp_avgs[i].ptr, exp_avg_sqs[i].ptr,
-                  None if vmax is None else vmax.ptr, param.data.size, state_steps[i], lr, beta1, beta2, eps,
-                  weight_decay, int(bool(amsgrad)), int(decoupled))
+        _device(param, grads[i], exp_avgs[i], exp_avg_sqs[i], max_exp_avg_sqs[i] if amsgrad else None)
+    pointers = ctypes.c_void_p * count
+    vmax = pointers(*[a.ptr for a in max_exp_avg_sqs]) if amsgrad else None
+    _hip.call('tt_adam_step_multi_f32', count, pointers(*[p.data.ptr for p in params]),
+              pointers(*[g.ptr for g in grads]), pointers(*[a.ptr for a in exp_avgs]),
+              pointers(*[a.ptr for a in exp_avg_sqs]), vmax, (ctypes.c_size_t * count)(*[p.data.size for p in params]),
+              (ctypes.c_int * count)(*state_steps), lr, beta1, beta2, eps, weight_decay, int(bool(amsgrad)),
+              int(decoupled))
 
 
 def adam(params, grads, exp_avgs, exp_avg_sqs, max_exp_avg_sqs, state_steps, amsgrad, beta1, beta2, lr,

@@ -149,3 +149,41 @@ def test_checkpoint_of_device_model_and_optimizer(tmp_path):
         o_.step()
     for (k, a), (_, b) in zip(net.state_dict().items(), net2.state_dict().items()):
         np.testing.assert_array_equal(a, b, err_msg=k)
+
+
+def test_many_parameters_in_one_group_take_several_launches():
+    """30 parameters of different sizes (more than one multi-tensor launch holds); one of them
+    only receives a gradient every other step, so its Adam step count lags behind."""
+    import pytortto_amd as tt
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(5)
+    shapes = [(1 + 7 * i, 3 + (i % 5)) for i in range(30)]
+    host = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    for kind in ('sgd', 'adam'):
+        params = [tt.nn.Parameter(tt.tensor(h.copy()).cuda().detach()) for h in host]
+        ref = [h.copy() for h in host]
+        if kind == 'sgd':
+            opt = tt.optim.SGD(params, lr=0.1, momentum=0.9, weight_decay=1e-3)
+            bufs = [None] * 30
+        else:
+            opt = tt.optim.Adam(params, lr=1e-2, betas=(0.9, 0.99))
+            m = [np.zeros_like(h) for h in host]
+            v = [np.zeros_like(h) for h in host]
+            steps = [0] * 30
+        for it in range(4):
+            grads = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+            live = [i for i in range(30) if not (i == 7 and it % 2)]
+            for i, p in enumerate(params):
+                p.grad = hiparray(grads[i]) if i in live else None
+            opt.step()
+            for i in live:
+                if kind == 'sgd':
+                    b = [bufs[i]]
+                    oracle.optim.sgd([ref[i]], [grads[i].copy()], b, 1e-3, 0.9, 0.1, 0, False)
+                    bufs[i] = b[0]
+                else:
+                    steps[i] += 1
+                    oracle.optim.adam([ref[i]], [grads[i]], [m[i]], [v[i]], [None], [steps[i]], False, 0.9, 0.99, 1e-2,
+                                      0, 1e-8)
+            for i in range(30):
+                np.testing.assert_array_equal(params[i].data.get(), ref[i], err_msg=f'{kind} step {it} parameter {i}')
