@@ -88,6 +88,18 @@ __device__ __forceinline__ void load_partials(const double2* __restrict__ partia
   b = wave_sum(p.y);
 }
 
+typedef float fx4 __attribute__((ext_vector_type(4)));
+// Streaming accesses: data that is not read again soon should not displace what is (the input x is
+// swept twice per pass) from the L2 and the memory-side cache.
+__device__ __forceinline__ float4 load_stream(const float4* p) {
+  const fx4 v = __builtin_nontemporal_load(reinterpret_cast<const fx4*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_stream(float4* p, const float4 o) {
+  const fx4 v = {o.x, o.y, o.z, o.w};
+  __builtin_nontemporal_store(v, reinterpret_cast<fx4*>(p));
+}
+
 constexpr int kStreamU = 8;   // float4 loads in flight per thread in the stream reduce kernel
 
 struct Geometry {
@@ -191,7 +203,9 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_stream(const float* __rest
       const float4 t = *reinterpret_cast<const float4*>(x + off);
       v[u] = ok ? t : fill;
       if constexpr (kBwd) {
-        const float4 q = *reinterpret_cast<const float4*>(dy + off);
+        // dy is streamed in both backward sweeps: x is read four times per training pass, dy twice,
+        // and at these sizes the memory-side cache cannot hold both
+        const float4 q = load_stream(reinterpret_cast<const float4*>(dy + off));
         gq[u] = ok ? q : zero;
       }
     }
@@ -307,13 +321,16 @@ __device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
         const int i = min(i0 + kThreads * u, hw4 - 1);   // clamped: out-of-range threads re-read, never store
-        v[u] = px[i];
-        gq[u] = kBwd ? pg[i] : v[u];
+        // backward: the last use of x and dy in the pass; forward: x is read again by the backward
+        v[u] = kBwd ? load_stream(px + i) : px[i];
+        gq[u] = kBwd ? load_stream(pg + i) : v[u];
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
         const int i = i0 + kThreads * u;
-        if (i < hw4) po[i] = apply4<kBwd>(v[u], gq[u], k);
+        if (i < hw4) {
+          store_stream(po + i, apply4<kBwd>(v[u], gq[u], k));
+        }
       }
     }
   }
@@ -332,16 +349,19 @@ __device__ __forceinline__ void sweep2_flat(const float* __restrict__ x, const f
     const uint32_t r = e - n * hwv;
     const size_t off = ((size_t)n * g.C + c) * g.HW + (size_t)r * VEC;
     if constexpr (VEC == 4) {
-      const float4 v = *reinterpret_cast<const float4*>(x + off);
+      const float4* px = reinterpret_cast<const float4*>(x + off);
+      const float4 v = kBwd ? load_stream(px) : *px;
       float4 gq = v;
-      if (kBwd) gq = *reinterpret_cast<const float4*>(dy + off);
-      *reinterpret_cast<float4*>(out + off) = apply4<kBwd>(v, gq, k);
+      if (kBwd) gq = load_stream(reinterpret_cast<const float4*>(dy + off));
+      store_stream(reinterpret_cast<float4*>(out + off), apply4<kBwd>(v, gq, k));
     } else {
-      const float v = x[off];
+      const float v = kBwd ? __builtin_nontemporal_load(x + off) : x[off];
+      float o;
       if (kBwd)
-        out[off] = fmaf(dy[off], k.k1, fmaf(v - k.m, k.k2, k.k0));
+        o = fmaf(__builtin_nontemporal_load(dy + off), k.k1, fmaf(v - k.m, k.k2, k.k0));
       else
-        out[off] = fmaf(v - k.m, k.k1, k.k0);
+        o = fmaf(v - k.m, k.k1, k.k0);
+      __builtin_nontemporal_store(o, out + off);
     }
   }
 }
