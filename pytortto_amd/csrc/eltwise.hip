@@ -28,6 +28,8 @@ template <int OP>
 __global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a, const float* __restrict__ b,
                                                     float* __restrict__ out, float alpha, size_t n) {
   constexpr bool kUseA = OP != kFill;
+  // results that are not accumulated in place stream out past the caches
+  constexpr bool kStreamOut = OP == kRelu || OP == kReluBwd || OP == kAdd || OP == kLeakyRelu || OP == kLeakyReluBwd;
   constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy || OP == kLeakyReluBwd;
   const size_t n4 = n >> 2;
   const size_t stride = (size_t)gridDim.x * kThreads;
@@ -39,7 +41,13 @@ __global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a,
     o.y = apply1<OP>(va.y, vb.y, alpha);
     o.z = apply1<OP>(va.z, vb.z, alpha);
     o.w = apply1<OP>(va.w, vb.w, alpha);
-    reinterpret_cast<float4*>(out)[i] = o;
+    if (kStreamOut) {
+      typedef float fx4 __attribute__((ext_vector_type(4)));
+      const fx4 ov = {o.x, o.y, o.z, o.w};
+      __builtin_nontemporal_store(ov, reinterpret_cast<fx4*>(out) + i);
+    } else {
+      reinterpret_cast<float4*>(out)[i] = o;
+    }
   }
   // tail (n % 4 elements)
   const size_t t = (n4 << 2) + (size_t)blockIdx.x * kThreads + threadIdx.x;

@@ -157,8 +157,8 @@ __global__ __launch_bounds__(kThreads) void maxpool_fwd_staged(const float* __re
         }
       }
     }
-    y[obase + o] = best;
-    tap[obase + o] = arg;
+    __builtin_nontemporal_store(best, y + obase + o);
+    __builtin_nontemporal_store(arg, tap + obase + o);
   }
 }
 
@@ -228,7 +228,9 @@ __global__ __launch_bounds__(kThreads) void maxpool_bwd_scatter(const float* __r
       v.y = __uint_as_float((uint32_t)a.y);
       v.z = __uint_as_float((uint32_t)c.x);
       v.w = __uint_as_float((uint32_t)c.y);
-      *reinterpret_cast<float4*>(dx + ibase + 4 * (size_t)k) = v;
+      typedef float fx4 __attribute__((ext_vector_type(4)));
+      const fx4 ov = {v.x, v.y, v.z, v.w};
+      __builtin_nontemporal_store(ov, reinterpret_cast<fx4*>(dx + ibase) + k);
     }
   } else {
     for (int e = threadIdx.x; e < count; e += kThreads) dx[ibase + e] = __uint_as_float((uint32_t)slot[e]);
