@@ -204,13 +204,9 @@ __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restr
 
 // ---- the GEMM kernel -----------------------------------------------------------------------------
 
-// Blocks are dealt round-robin to the 8 XCDs; give each XCD a contiguous range of tiles, row
-// tiles fastest, so blocks that share a pixel tile (same gathered operand) share an L2.
-__device__ __forceinline__ int xcd_remap(int b, int nb) {
-  const int q = nb >> 3, rem = nb & 7;
-  const int xcd = b & 7, idx = b >> 3;
-  return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
-}
+// Blocks are dealt round-robin to the 8 XCDs; tt::xcd_remap gives each XCD a contiguous range of
+// tiles, row tiles fastest, so blocks that share a pixel tile (same gathered operand) share an L2.
+using tt::xcd_remap;
 
 constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2;
 constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format

@@ -112,9 +112,18 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
-  const int g = blockIdx.y, split = blockIdx.z;
-  const int i0 = (blockIdx.x % p.tilesI) * BM;
-  const int j0 = (blockIdx.x / p.tilesI) * BN;
+  // The tiles of one reduction split read the same pixels of x and dy: with one group, splits are
+  // dealt to the XCDs in contiguous runs so that those tiles share an L2 instead of each XCD
+  // fetching every split's pixels.
+  const int g = blockIdx.y;
+  int tile = blockIdx.x, split = blockIdx.z;
+  if (gridDim.y == 1) {
+    const int v = tt::xcd_remap((int)(blockIdx.x + gridDim.x * blockIdx.z), (int)(gridDim.x * gridDim.z));
+    split = v / (int)gridDim.x;
+    tile = v - split * (int)gridDim.x;
+  }
+  const int i0 = (tile % p.tilesI) * BM;
+  const int j0 = (tile / p.tilesI) * BN;
 
   if (tid < BN) {
     const int j = j0 + tid;

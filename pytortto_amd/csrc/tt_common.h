@@ -46,6 +46,14 @@ __device__ __forceinline__ uint32_t fd_div(uint32_t n, const FastDiv& f) {
   return (uint32_t)(((uint64_t)__umulhi(n, f.mul) + n) >> f.shift);
 }
 
+// Blocks are dealt round-robin to the 8 XCDs (each with its own L2) in launch order.  Maps block b
+// of nb to a work index such that every XCD receives one contiguous range of work indices.
+__device__ __forceinline__ int xcd_remap(int b, int nb) {
+  const int q = nb >> 3, rem = nb & 7;
+  const int xcd = b & 7, idx = b >> 3;
+  return (xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q) + idx;
+}
+
 }  // namespace tt
 
 #define TT_HIP(expr)                                                      \
