@@ -769,14 +769,19 @@ bool wants_stream_k(long long tiles, int chunks, int groups) {
 
 // 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
 // CUs idle or unevenly loaded the reduction is split stream-K fashion; if it is too short for
-// that, 64x64 tiles raise the block count instead.
-TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k = true) {
+// that, 64x64 tiles raise the block count instead.  `small` asks for 64x64 tiles outright: many
+// light blocks (four or five resident per CU) balance better and need no fix-up stage where a
+// tile's reduction is short (plain matrix products with at most 32 chunks) or where several
+// short launches share a grid (the stride-parity classes of an input gradient).
+TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k = true, bool small = false) {
   TileChoice t;
   t.bm = I <= 64 ? 64 : 128;
   t.bn = I <= 64 ? 256 : 128;
+  if (small && groups == 1) { t.bm = 64; t.bn = 64; }
   if (const char* e = getenv("TT_IGEMM_TILE")) {   // tuning knob: 0 = 128x128, 1 = 64x256
     if (e[0] == '0') { t.bm = 128; t.bn = 128; }
     if (e[0] == '1') { t.bm = 64; t.bn = 256; }
+    if (e[0] == '2') { t.bm = 64; t.bn = 64; }
   }
   t.sk_blocks = 0;
   const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
@@ -968,7 +973,8 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   const int Kred = Cg * R * S;
   const int M = N * P * Q;
   const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
-  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ);
+  const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
+  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ, true, plain && KQ / kBKQ <= 32);
   const int Ipad = ceil_div(Kg, t.bm) * t.bm;
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
@@ -1156,7 +1162,9 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       if (Kred == 0 && prefilled) continue;
       const int M = N * U * V;
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
-      const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k);
+      const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
+      const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k,
+                                       (plain && KQ / kBKQ <= 32) || !allow_stream_k);
       const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
