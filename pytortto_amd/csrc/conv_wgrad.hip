@@ -488,6 +488,11 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   int bm = 128, bn = 128;
   if (Kg <= 64) bm = 64;
   if (J <= 64) bn = 64;
+  // 64 columns where 128 would be badly filled (the 7x7 stem: J = 147), and for 1x1 layers: twice
+  // the tiles means half the reduction splits, so half the partial sums to write and add up
+  // (measured on the ResNet-50 shapes: 4-7 % faster there, slower for 3x3 layers).
+  if (J % 128 != 0 && J % 128 <= 64) bn = 64;
+  if (R == 1 && S == 1 && Kg >= 128) bn = 64;
   const int tilesI = ceil_div(Kg, bm), tilesJ = ceil_div(J, bn);
   const long long tiles = (long long)tilesI * tilesJ * groups;
   const int chunks = ceil_div(M, kBK);
