@@ -126,8 +126,8 @@ template <int K>
 __global__ __launch_bounds__(kThreads) void maxpool_fwd_staged(const float* __restrict__ x, float* __restrict__ y,
                                                                int* __restrict__ tap, Pool g, Band b) {
   __shared__ __align__(16) float lds[kStageFloats + 8];
-  const int nc = blockIdx.y;
-  const int p0 = blockIdx.x * b.rows;
+  const int nc = blockIdx.x;
+  const int p0 = blockIdx.y * b.rows;
   const int p1 = min(g.P, p0 + b.rows);
   const int kh = K ? K : g.kh, kw = K ? K : g.kw;
   const int h_lo = max(0, p0 * g.sh - g.ph);
@@ -173,8 +173,8 @@ __global__ __launch_bounds__(kThreads) void maxpool_bwd_scatter(const float* __r
                                                                 const int* __restrict__ tap,
                                                                 float* __restrict__ dx, Pool g, Band b) {
   __shared__ __align__(16) unsigned long long slot[kScatterSlots];
-  const int nc = blockIdx.y;
-  const int h0 = blockIdx.x * b.rows;
+  const int nc = blockIdx.x;
+  const int h0 = blockIdx.y * b.rows;
   const int h1 = min(g.H, h0 + b.rows);
   const int rows = h1 - h0;
   const int count = rows * g.W;
@@ -285,9 +285,9 @@ int tt_maxpool2d_fwd_f32(const float* x, float* y, int* tap, int NC, int H, int 
   // output rows per block: as many as keep the input rows they need within the LDS stage
   const long long first = (long long)(kh - 1) * dh + 1;          // input rows of one output row
   const long long fit = ((long long)kStageFloats / W - first) / sh + 1;
-  if ((long long)first * W <= kStageFloats && NC <= 65535 && fit >= 1) {
+  if ((long long)first * W <= kStageFloats && fit >= 1) {
     Band b = make_band(g, (int)(fit < P ? fit : P), 32);
-    const dim3 grid((P + b.rows - 1) / b.rows, NC);
+    const dim3 grid(NC, (P + b.rows - 1) / b.rows);       // planes on x: their number has no 16-bit limit
     if (kh == 3 && kw == 3) maxpool_fwd_staged<3><<<grid, kThreads, 0, tt::stream()>>>(x, y, tap, g, b);
     else if (kh == 2 && kw == 2) maxpool_fwd_staged<2><<<grid, kThreads, 0, tt::stream()>>>(x, y, tap, g, b);
     else maxpool_fwd_staged<0><<<grid, kThreads, 0, tt::stream()>>>(x, y, tap, g, b);
@@ -308,9 +308,9 @@ int tt_maxpool2d_bwd_f32(const float* dy, const int* tap, float* dx, int NC, int
   tt::ProfScope prof(TT_PROF_MAXPOOL_BWD);
   // input rows per block: one 8-byte LDS slot per pixel of the band
   const int fit = kScatterSlots / W;
-  if (NC <= 65535 && fit >= 1) {
+  if (fit >= 1) {
     Band b = make_band(g, fit < H ? fit : H, 32);
-    const dim3 grid((H + b.rows - 1) / b.rows, NC);
+    const dim3 grid(NC, (H + b.rows - 1) / b.rows);
     maxpool_bwd_scatter<<<grid, kThreads, 0, tt::stream()>>>(dy, tap, dx, g, b);
   } else {
     maxpool_bwd<<<grid_for(total), kThreads, 0, tt::stream()>>>(dy, tap, dx, g, total);

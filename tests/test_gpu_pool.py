@@ -50,6 +50,10 @@ def test_max_pool_rows_too_wide_for_the_lds_stage():
     _run_pool((1, 2, 40, 700, (5, 2), (1, 1), (2, 1), (1, 1), False), seed=12, ties=True)   # one output row per block
 
 
+def test_max_pool_more_than_65535_planes():
+    _run_pool((1100, 60, 4, 6, (2, 2), (2, 2), (0, 0), (1, 1), False), seed=13, ties=True)
+
+
 def test_max_pool_full_size_properties():
     """[64,64,112,112], 3x3 stride 2 padding 1 (the ResNet-50 stem pooling): with dy = y every
     assigned gradient equals the input at that pixel, each window's maximum is found in the
