@@ -281,7 +281,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this path runs on exactly one GPU (asked for --gpus {args.gpus}); '
-              f'nothing in it is sharded, see DESIGN.md for how it would be', file=sys.stderr)
+              f'nothing in it is sharded (it would shard by batch: one all-reduce of the weight gradients, and of the '
+              f'per-channel BatchNorm moments between the two sweeps)', file=sys.stderr)
         sys.exit(2)
 
     from pytortto_amd import _hip
