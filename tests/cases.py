@@ -39,3 +39,44 @@ POOL_CASES = [
     (3, 1, 5, 9, (5, 3), (1, 3), (2, 1), (1, 1), False),      # tall kernel
     (2, 2, 8, 8, (2, 2), (3, 3), (0, 0), (1, 1), False),      # stride > kernel: uncovered pixels
 ]
+
+
+def random_pool_cases(count, seed):
+    """Seeded random pooling geometries (kernel, stride, padding <= kernel / 2, dilation, ceil_mode)."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        ks = (int(rng.integers(1, 6)), int(rng.integers(1, 6)))
+        st = (int(rng.integers(1, 5)), int(rng.integers(1, 5)))
+        pd = (int(rng.integers(0, ks[0] // 2 + 1)), int(rng.integers(0, ks[1] // 2 + 1)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        cm = bool(rng.integers(0, 2))
+        h, w = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        if min(oracle.pool_output_size(h, ks[0], st[0], pd[0], dl[0], cm),
+               oracle.pool_output_size(w, ks[1], st[1], pd[1], dl[1], cm)) < 1:
+            continue
+        cases.append((int(rng.integers(1, 4)), int(rng.integers(1, 6)), h, w, ks, st, pd, dl, cm))
+    return cases
+
+
+def random_conv_cases(count, seed):
+    """Seeded random geometries: every combination of stride, padding, dilation and groups the
+    validation admits, with sizes that are not multiples of any tile."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        g = int(rng.choice([1, 1, 1, 2, 3, 4]))
+        c, k = g * int(rng.integers(1, 24)), g * int(rng.integers(1, 24))
+        r, s = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pd = (int(rng.integers(0, 4)), int(rng.integers(0, 4)))
+        h, w = int(rng.integers(1, 23)), int(rng.integers(1, 23))
+        n = int(rng.integers(1, 6))
+        if h + 2 * pd[0] < dl[0] * (r - 1) + 1 or w + 2 * pd[1] < dl[1] * (s - 1) + 1:
+            continue
+        cases.append((n, c, h, w, k, r, s, st, pd, dl, g))
+    return cases

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from tests.cases import CONV_CASES, CONVT_CASES
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases
 
 pytestmark = pytest.mark.gpu
 
@@ -152,3 +152,9 @@ def test_conv_rejects_bad_arguments():
         ops.conv2d_fwd(x, w, None, (1, 1), (0, 0), (1, 1), 3)      # channels not divisible by groups
     with pytest.raises(RuntimeError):
         ops.conv2d_fwd(x, w, None, (1, 1), (0, 0), (2, 2), 1)      # dilated kernel larger than the input
+
+
+@pytest.mark.parametrize('case', random_conv_cases(60, 2024), ids=lambda c: 'n%d_c%d_%dx%d_k%d_%dx%d_s%s_p%s_d%s_g%d' % (
+    c[0], c[1], c[2], c[3], c[4], c[5], c[6], '%d%d' % c[7], '%d%d' % c[8], '%d%d' % c[9], c[10]))
+def test_conv_random_geometries(case):
+    _run_conv(case, seed=5)

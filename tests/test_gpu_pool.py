@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from tests.cases import POOL_CASES
+from tests.cases import POOL_CASES, random_pool_cases
 
 pytestmark = pytest.mark.gpu
 
@@ -142,3 +142,9 @@ def test_relu_keeps_nan():
     x = np.array([np.nan, -1.0, 0.0, 2.0, -0.0], np.float32)
     y = ops.relu_fwd(hiparray(x)).get()
     np.testing.assert_array_equal(y, oracle.relu_forward(x))
+
+
+@pytest.mark.parametrize('case', random_pool_cases(60, 77), ids=lambda c: '%dx%d_k%d%d_s%d%d_p%d%d_d%d%d_%s' % (
+    c[2], c[3], *c[4], *c[5], *c[6], *c[7], 'ceil' if c[8] else 'floor'))
+def test_max_pool_random_geometries(case):
+    _run_pool(case, seed=14, ties=True)

@@ -7,7 +7,7 @@ import torch.nn.functional as TF
 
 import oracle
 from tests import brute
-from tests.cases import POOL_CASES
+from tests.cases import POOL_CASES, random_pool_cases
 
 
 def _data(case, seed=0, ties=False):
@@ -112,3 +112,19 @@ def test_relu_and_leaky_relu_closed_forms_and_torch():
     yt.backward(torch.from_numpy(g))
     np.testing.assert_array_equal(oracle.relu_forward(x), yt.detach().numpy())
     np.testing.assert_array_equal(oracle.relu_backward(g, oracle.relu_forward(x)), xt.grad.numpy())
+
+
+@pytest.mark.parametrize('case', random_pool_cases(60, 77))
+def test_max_pool_random_geometries_against_torch(case):
+    """Values and arg-max positions against torch on the geometries the GPU sweep uses (rounded
+    inputs, so ties are everywhere); windows that lie wholly in the padding are left out of the
+    index comparison (torch reports an index there, the reference's tap points into the padding)."""
+    x, _ = _data(case, seed=3, ties=True)
+    ks, st, pd, dl, cm = case[4:]
+    y, pos = oracle.max_pool2d(x, ks, st, pd, dl, cm)
+    yt, it = TF.max_pool2d(torch.from_numpy(x), ks, st, pd, dl, ceil_mode=cm, return_indices=True)
+    assert y.shape == tuple(yt.shape)
+    np.testing.assert_array_equal(y, yt.numpy())
+    hh, ww = _where_from_pos(pos, case)
+    inside = (hh >= 0) & (hh < x.shape[2]) & (ww >= 0) & (ww < x.shape[3])
+    np.testing.assert_array_equal((hh * x.shape[3] + ww)[inside], it.numpy()[inside])
