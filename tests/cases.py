@@ -80,3 +80,27 @@ def random_conv_cases(count, seed):
             continue
         cases.append((n, c, h, w, k, r, s, st, pd, dl, g))
     return cases
+
+
+def random_convt_cases(count, seed):
+    """Seeded random transposed-convolution geometries with output_padding < stride: what the
+    reference's own `output_size` path can produce (nn/modules/conv.py:137-153); beyond that its
+    backward returns an input gradient larger than the input."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        g = int(rng.choice([1, 1, 2, 3]))
+        ci, co = g * int(rng.integers(1, 16)), g * int(rng.integers(1, 16))
+        r, s = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pd = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        op = (int(rng.integers(0, st[0])), int(rng.integers(0, st[1])))
+        h, w = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        ho = (h - 1) * st[0] - 2 * pd[0] + dl[0] * (r - 1) + op[0] + 1
+        wo = (w - 1) * st[1] - 2 * pd[1] + dl[1] * (s - 1) + op[1] + 1
+        if ho < 1 or wo < 1:
+            continue
+        cases.append((int(rng.integers(1, 5)), ci, h, w, co, r, s, st, pd, op, dl, g))
+    return cases

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
 
 pytestmark = pytest.mark.gpu
 
@@ -113,7 +113,7 @@ CONVT_TILE_CASES = [
 ]
 
 
-@pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES)
+@pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES + random_convt_cases(40, 99))
 def test_conv_transpose_forward_backward(case):
     from pytortto_amd import ops
     from pytortto_amd.xparray import hiparray

@@ -7,7 +7,7 @@ import torch.nn.functional as TF
 
 import oracle
 from tests import brute
-from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
 
 
 def _rand(shape, rng, dtype=np.float64):
@@ -140,6 +140,24 @@ def test_conv_transpose_matches_definition_and_torch(case):
     lhs = float((y_def - b[None, :, None, None]).ravel() @ gy.ravel())
     assert abs(lhs - float((x * dx).sum())) <= 1e-10 * max(1.0, abs(lhs))
     assert abs(lhs - float((w * dw).sum())) <= 1e-10 * max(1.0, abs(lhs))
+
+
+@pytest.mark.parametrize('case', random_convt_cases(40, 99))
+def test_conv_transpose_random_geometries_against_torch(case):
+    n, ci, h, w_, co, r, s, st, pd, op, dl, g = case
+    rng = np.random.default_rng(8)
+    x, w, b = _rand((n, ci, h, w_), rng), _rand((ci, co // g, r, s), rng), _rand((co,), rng)
+    y = oracle.transposed_convolution_forward(x, w, b, st, pd, op, dl, g)
+    xt, wt, bt = (torch.tensor(a, requires_grad=True) for a in (x, w, b))
+    yt = TF.conv_transpose2d(xt, wt, bt, st, pd, op, g, dl)
+    assert y.shape == tuple(yt.shape)
+    np.testing.assert_allclose(y, yt.detach().numpy(), rtol=1e-11, atol=1e-11)
+    gy = _rand(y.shape, rng)
+    yt.backward(torch.tensor(gy))
+    dx, dw, db = oracle.transposed_convolution_backward(gy, x, w, st, pd, dl, g)
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(dw, wt.grad.numpy(), rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(db, bt.grad.numpy(), rtol=1e-11, atol=1e-11)
 
 
 def test_conv_transpose_output_size_formula():
