@@ -196,3 +196,20 @@ def test_bn_benchmark_shapes_full_size(shape):
     scale = float(np.abs(dx).sum(axis, dtype=np.float64).max())
     assert np.abs(dx.sum(axis, dtype=np.float64)).max() <= 1e-5 * scale
     assert np.abs((dx * xhat).sum(axis)).max() <= 1e-4 * scale          # exact only up to O(eps / var)
+
+
+def _random_bn_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        n, c = int(rng.integers(1, 40)), int(rng.integers(1, 70))
+        h, w = int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        if n * h * w < 2:
+            continue
+        shapes.append((n, c, h, w))
+    return shapes
+
+
+@pytest.mark.parametrize('shape', _random_bn_shapes(40, 31), ids=lambda s: '%dx%dx%dx%d' % s)
+def test_bn_random_shapes(shape):
+    test_bn_train_fwd_bwd_matches_oracle(shape)
