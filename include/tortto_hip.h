@@ -143,6 +143,21 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
                   const float* save_mean, const float* save_var_eps, const float* save_sd,
                   float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
 
+/* ---- workspace queries (no counterpart in the reference) -------------------------------------- */
+
+/* Bytes of library workspace (repacked weights, index tables, partial sums) the corresponding call
+ * asks for with the same geometry arguments; the library grows its workspace to the largest
+ * request seen.  Same argument checks as the calls; nothing is launched or allocated.  The small
+ * per-geometry tables the library caches separately (index tables, 16 bytes per output pixel for
+ * the weight gradient) are not included. */
+int tt_workspace_size_conv2d_fwd_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S,
+                                     int sh, int sw, int ph, int pw, int dh, int dw, int groups);
+int tt_workspace_size_conv2d_dgrad_f32(size_t* bytes, int N, int C, int Hx, int Wx, int K, int R, int S,
+                                       int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q);
+int tt_workspace_size_conv2d_wgrad_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S,
+                                       int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q);
+int tt_workspace_size_bn_f32(size_t* bytes, int N, int C, int HW);   /* training forward and backward alike */
+
 /* ---- MaxPool2d (autograd/grad_nn.py:784-864) ------------------------------------------------ */
 
 /* x: [NC, H, W] planes (N*C of them), y and tap: [NC, P, Q].  Windows are taken over x padded

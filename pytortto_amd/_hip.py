@@ -38,6 +38,10 @@ PROTOTYPES = {
     'tt_conv2d_dgrad_f32': [_P, _P, _P, _P] + [_I] * 16,
     'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
     'tt_channel_sum_f32': [_P, _P, _I, _I, _I],
+    'tt_workspace_size_conv2d_fwd_f32': [POINTER(c_size_t)] + [_I] * 14,
+    'tt_workspace_size_conv2d_dgrad_f32': [POINTER(c_size_t)] + [_I] * 16,
+    'tt_workspace_size_conv2d_wgrad_f32': [POINTER(c_size_t)] + [_I] * 16,
+    'tt_workspace_size_bn_f32': [POINTER(c_size_t), _I, _I, _I],
     'tt_bn_fwd_train_f32': [_P] * 11 + [c_double, c_double, _I, _I, _I],
     'tt_bn_fwd_eval_f32': [_P] * 9 + [c_double, _I, _I, _I],
     'tt_bn_bwd_f32': [_P] * 9 + [_I, _I, _I],

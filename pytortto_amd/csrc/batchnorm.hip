@@ -680,4 +680,16 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
   return 0;
 }
 
+// Workspace of tt_bn_fwd_train_f32 and tt_bn_bwd_f32 alike: one double2 partial per channel and
+// reduction split of the first sweep.
+int tt_workspace_size_bn_f32(size_t* bytes, int N, int C, int HW) {
+  TT_REQUIRE(bytes, "tt_workspace_size_bn_f32: null result pointer");
+  if (check_shape("tt_workspace_size_bn_f32", N, C, HW)) return -1;
+  Geometry gr;
+  int rmode;
+  plan_reduce(N, C, HW, &gr, &rmode);
+  *bytes = sizeof(double2) * (size_t)C * gr.splits;
+  return 0;
+}
+
 }  // extern "C"

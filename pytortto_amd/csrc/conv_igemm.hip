@@ -959,8 +959,9 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 extern "C" {
 
-int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
-                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
+// `size_only`: report the workspace bytes this call would ask the library for and do nothing else.
+static int conv2d_fwd(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
+                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, size_t* size_only) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
   const int P = (H + 2 * ph - dh * (R - 1) - 1) / sh + 1;
@@ -979,6 +980,10 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
   const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
+  if (size_only) {
+    *size_only = wp_bytes + tab_bytes + sk_workspace_bytes();
+    return 0;
+  }
   void* ws;
   if (tt::workspace(wp_bytes + tab_bytes + sk_workspace_bytes(), &ws)) return -1;
   floatx4* wp = (floatx4*)ws;
@@ -1021,9 +1026,9 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes + tab_bytes));
 }
 
-int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
+static int conv2d_dgrad(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
                         int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
-                        int Q) {
+                        int Q, size_t* size_only) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
   if (check_common("tt_conv2d_dgrad_f32", N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
@@ -1068,6 +1073,10 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
       const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)KQ * Ipad, 256);
       const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
       const size_t row_bytes = align_up(sizeof(int4) * (size_t)I, 256);
+      if (size_only) {
+        *size_only = wp_bytes + tab_bytes + row_bytes;
+        return 0;
+      }
       void* ws;
       if (tt::workspace(wp_bytes + tab_bytes + row_bytes, &ws)) return -1;
       floatx4* wp = (floatx4*)ws;
@@ -1102,6 +1111,10 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
   const int IpadMax = ceil_div(Cg, 128) * 128;
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQmax * IpadMax, 256);
   const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQmax * 4, 256);
+  if (size_only) {
+    *size_only = (wp_bytes + tab_bytes) * classes + sk_workspace_bytes();
+    return 0;
+  }
   void* ws;
   if (tt::workspace((wp_bytes + tab_bytes) * classes + sk_workspace_bytes(), &ws)) return -1;
   floatx4* sk_partial = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * classes);
@@ -1226,6 +1239,35 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
     if (launch_igemm_multi(multi, groups, multi_tile, TT_PROF_CONV_IGEMM_DGRAD)) return -1;
   }
   return 0;
+}
+
+int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
+                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
+  return conv2d_fwd(x, w, bias, y, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr);
+}
+
+int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
+                        int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
+                        int Q) {
+  return conv2d_dgrad(dy, w, bias, dx, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q, nullptr);
+}
+
+// The queries run the same argument checks and planning as the calls themselves, with placeholder
+// tensor pointers that are never dereferenced, and stop where the call would ask for the workspace.
+int tt_workspace_size_conv2d_fwd_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S, int sh, int sw,
+                                     int ph, int pw, int dh, int dw, int groups) {
+  TT_REQUIRE(bytes, "tt_workspace_size_conv2d_fwd_f32: null result pointer");
+  const float* in = reinterpret_cast<const float*>(uintptr_t(256));
+  return conv2d_fwd(in, in, nullptr, const_cast<float*>(in), N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups,
+                    bytes);
+}
+
+int tt_workspace_size_conv2d_dgrad_f32(size_t* bytes, int N, int C, int Hx, int Wx, int K, int R, int S, int sh,
+                                       int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q) {
+  TT_REQUIRE(bytes, "tt_workspace_size_conv2d_dgrad_f32: null result pointer");
+  const float* in = reinterpret_cast<const float*>(uintptr_t(256));
+  return conv2d_dgrad(in, in, nullptr, const_cast<float*>(in), N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups,
+                      P, Q, bytes);
 }
 
 }  // extern "C"

@@ -468,8 +468,9 @@ void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStre
 
 extern "C" {
 
-int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
-                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+// `size_only`: report the workspace bytes this call would ask the library for and do nothing else.
+static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
+                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q, size_t* size_only) {
   TT_REQUIRE_INIT();
   const char* fn = "tt_conv2d_wgrad_f32";
   TT_REQUIRE(x && dy && dw, "%s: null tensor pointer", fn);
@@ -510,6 +511,10 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
   splits = ceil_div(chunks, cps);
 
   const size_t elems = (size_t)groups * Kg * J;
+  if (size_only) {
+    *size_only = splits > 1 ? sizeof(float) * elems * splits : 0;
+    return 0;
+  }
   float* target = dw;
   if (splits > 1) {
     void* ws;
@@ -566,6 +571,19 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C
     TT_LAUNCH_CHECK();
   }
   return 0;
+}
+
+int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
+                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+  return conv2d_wgrad(x, dy, dw, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw_, groups, P, Q, nullptr);
+}
+
+int tt_workspace_size_conv2d_wgrad_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S, int sh, int sw,
+                                       int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+  TT_REQUIRE(bytes, "tt_workspace_size_conv2d_wgrad_f32: null result pointer");
+  const float* in = reinterpret_cast<const float*>(uintptr_t(256));   // placeholder, never dereferenced
+  return conv2d_wgrad(in, in, const_cast<float*>(in), N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw_, groups, P, Q,
+                      bytes);
 }
 
 }  // extern "C"

@@ -254,3 +254,47 @@ def test_device_memory_is_pooled_and_released():
     b = hiparray(np.zeros((256, 256), np.float32))
     assert b.ptr == ptr                       # same size class: the pooled block is reused
     _hip.call('tt_empty_cache')
+
+
+def test_workspace_queries_bound_what_the_calls_request():
+    """tt_workspace_size_* report what a call asks the library for: after tt_empty_cache() the
+    workspace grows to at least that (the library adds a quarter of head room), never before."""
+    import ctypes
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+
+    def workspace_now():
+        used, pooled, ws = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+        _hip.call('tt_mem_stats', ctypes.byref(used), ctypes.byref(pooled), ctypes.byref(ws))
+        return ws.value
+
+    def query(name, *args):
+        out = ctypes.c_size_t()
+        _hip.call(name, ctypes.byref(out), *args)
+        return out.value
+
+    n, c, h, k, r, st, pd = 8, 96, 28, 160, 3, 2, 1
+    q = (h + 2 * pd - r) // st + 1
+    geo = (n, c, h, h, k, r, r, st, st, pd, pd, 1, 1, 1)
+    rng = np.random.default_rng(0)
+    x = hiparray(rng.standard_normal((n, c, h, h), dtype=np.float32))
+    w = hiparray(rng.standard_normal((k, c, r, r), dtype=np.float32))
+    g = hiparray(rng.standard_normal((n, k, q, q), dtype=np.float32))
+    sizes = {'fwd': query('tt_workspace_size_conv2d_fwd_f32', *geo),
+             'dgrad': query('tt_workspace_size_conv2d_dgrad_f32', *geo, q, q),
+             'wgrad': query('tt_workspace_size_conv2d_wgrad_f32', *geo, q, q),
+             'bn': query('tt_workspace_size_bn_f32', n, k, q * q)}
+    assert all(v > 0 for v in sizes.values()), sizes
+    runs = {'fwd': lambda: ops.conv2d_fwd(x, w, None, (st, st), (pd, pd), (1, 1), 1),
+            'dgrad': lambda: ops.conv2d_dgrad(g, w, None, (h, h), (st, st), (pd, pd), (1, 1), 1),
+            'wgrad': lambda: ops.conv2d_wgrad(x, g, (k, c, r, r), (st, st), (pd, pd), (1, 1), 1),
+            'bn': lambda: ops.bn_fwd_train(g, None, None, None, None, 0.1, 1e-5)}
+    for name, run in runs.items():
+        _hip.synchronize()
+        _hip.call('tt_empty_cache')
+        assert workspace_now() == 0
+        run()
+        got = workspace_now()
+        assert sizes[name] <= got <= 2 * sizes[name] + (1 << 20), (name, sizes[name], got)
+    with pytest.raises(RuntimeError, match='not divisible by groups'):
+        query('tt_workspace_size_conv2d_fwd_f32', n, c, h, h, k, r, r, st, st, pd, pd, 1, 1, 7)
