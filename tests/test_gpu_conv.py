@@ -158,3 +158,31 @@ def test_conv_rejects_bad_arguments():
     c[0], c[1], c[2], c[3], c[4], c[5], c[6], '%d%d' % c[7], '%d%d' % c[8], '%d%d' % c[9], c[10]))
 def test_conv_random_geometries(case):
     _run_conv(case, seed=5)
+
+
+@pytest.mark.parametrize('case', [
+    (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # stream-K forward and input gradient, split weight gradient
+    (8, 256, 14, 14, 256, 3, 3, (2, 2), (1, 1), (1, 1), 1),     # parity classes in one grid
+    (16, 256, 14, 14, 1024, 1, 1, (1, 1), (0, 0), (1, 1), 1),   # 64x64 tiles
+])
+def test_conv_is_bit_reproducible(case):
+    """Split reductions are added in a fixed order: the same call gives the same bits every time."""
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(6)
+    x = hiparray(rng.standard_normal((n, c, h, w_), dtype=np.float32))
+    w = hiparray(rng.standard_normal((k, c // g, r, s), dtype=np.float32))
+    p = (h + 2 * pd[0] - dl[0] * (r - 1) - 1) // st[0] + 1
+    q = (w_ + 2 * pd[1] - dl[1] * (s - 1) - 1) // st[1] + 1
+    gy = hiparray(rng.standard_normal((n, k, p, q), dtype=np.float32))
+
+    def once():
+        return (ops.conv2d_fwd(x, w, None, st, pd, dl, g).get(), ops.conv2d_dgrad(gy, w, None, (h, w_), st, pd, dl, g).get(),
+                ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get())
+
+    first = once()
+    ops.conv2d_fwd(hiparray(rng.standard_normal((4, 8, 9, 9), dtype=np.float32)),           # other work in between
+                   hiparray(rng.standard_normal((8, 8, 3, 3), dtype=np.float32)), None, (1, 1), (1, 1), (1, 1), 1)
+    for a, b in zip(first, once()):
+        np.testing.assert_array_equal(a, b)
