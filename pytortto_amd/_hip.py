@@ -26,6 +26,8 @@ PROTOTYPES = {
     'tt_memcpy_d2d': [_P, _P, c_size_t],
     'tt_memset': [_P, _I, c_size_t],
     'tt_sync': [],
+    'tt_set_conv_math': [_I],
+    'tt_get_conv_math': [POINTER(c_int)],
     'tt_event_create': [POINTER(c_void_p)],
     'tt_event_record': [_P],
     'tt_event_elapsed_ms': [_P, _P, POINTER(c_float)],
@@ -161,6 +163,24 @@ def probe_hbm(nbytes=2 << 30):
     rd, cp = c_double(), c_double()
     call('tt_probe_hbm_f32', nbytes, ctypes.byref(rd), ctypes.byref(cp))
     return rd.value, cp.value
+
+
+CONV_MATH = {'f32': 0, 'bf16': 1}
+
+
+def set_conv_math(mode):
+    """Matrix arithmetic of convolution forward / input gradient: 'f32' (default, the mode that meets
+    the reference's tolerances) or 'bf16' (operands rounded to bfloat16 inside the kernel, float32
+    accumulation; tensors stay float32)."""
+    if mode not in CONV_MATH:
+        raise ValueError(f"conv math must be one of {sorted(CONV_MATH)}, got {mode!r}")
+    call('tt_set_conv_math', CONV_MATH[mode])
+
+
+def get_conv_math():
+    mode = c_int()
+    call('tt_get_conv_math', ctypes.byref(mode))
+    return {v: k for k, v in CONV_MATH.items()}[mode.value]
 
 
 def synchronize():

@@ -26,6 +26,10 @@
 // reduction index only moves a scalar offset, and padding is left to the buffer range check
 // (a lane whose tap falls outside the image gets bit 31 of its offset set, two VALU
 // instructions per element, and reads 0).
+//
+// Optional reduced-precision variant (tt_set_conv_math(TT_CONV_MATH_BF16)): the same kernels with
+// the operands rounded to bfloat16 after the LDS read and contracted by v_mfma_f32_32x32x16_bf16,
+// float32 accumulation, float32 tensors in memory.
 #include <cstdlib>
 #include <map>
 
@@ -35,6 +39,7 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
 constexpr int kBKQ = 4;          // k-quads per chunk (BK = 16)
@@ -226,7 +231,7 @@ __device__ __forceinline__ void wait_loads() {
 
 // The kernel body: `block_x` is the block's index among the blocks of launch `p` (a launch may
 // be one of several that share a grid, see igemm_multi_f32).
-template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT, bool BF>
 __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
@@ -453,7 +458,39 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   // sched_barrier pins this order; the compiler otherwise sinks the loads below the MFMAs.
   constexpr int T = 8 * MT * NT;
   auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
-    if constexpr (T >= 32) {
+    if constexpr (BF) {
+      // bf16 matrix instructions: one v_mfma_f32_32x32x16_bf16 per accumulator contracts the whole
+      // chunk (a lane's two quads are its eight k values, the same ones for both operands), so a
+      // chunk's matrix time is a sixteenth of the fp32 one and there is no shadow to weave the
+      // loads into; more resident blocks hide them instead.  Operands are rounded to bf16
+      // (nearest even) after the LDS read; accumulation stays fp32.
+      load_all(nchunk);
+      __builtin_amdgcn_sched_barrier(0);
+      bf16x8 a[MT], b[NT];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int x = 0; x < MT; ++x) {
+          a[x][j] = (__bf16)opA[set][0][x][j];
+          a[x][4 + j] = (__bf16)opA[set][1][x][j];
+        }
+#pragma unroll
+        for (int y = 0; y < NT; ++y) {
+          b[y][j] = (__bf16)opB[set][0][y][j];
+          b[y][4 + j] = (__bf16)opB[set][1][y][j];
+        }
+      }
+#pragma unroll
+      for (int x = 0; x < MT; ++x)
+#pragma unroll
+        for (int y = 0; y < NT; ++y)
+          acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      store_all(set ^ 1);
+      __syncthreads();
+      read_ops(set ^ 1, set ^ 1);
+      load_tab(nnchunk);
+    } else if constexpr (T >= 32) {
       constexpr int kStore = T - 8, kSync = T - 4;
       constexpr int nL = GEMM ? GR : nB;   // load steps of the gathered operand
       static_assert(nL + A_ITEMS <= kStore && kStore + B_ITEMS + A_ITEMS - 1 <= kSync, "schedule does not fit");
@@ -673,7 +710,12 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
 
 template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
-  igemm_body<WM, WN, MT, NT, SK, MODE, AT>(p, (int)blockIdx.x);
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT, false>(p, (int)blockIdx.x);
+}
+// The same launch on bf16 matrix instructions (tt_set_conv_math); three blocks per CU.
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
+__global__ __launch_bounds__(kThreads, 3) void igemm_bf16(const Igemm p) {
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT, true>(p, (int)blockIdx.x);
 }
 
 // Several data-parallel launches in one grid (the stride-parity classes of a strided input
@@ -689,7 +731,13 @@ template <int WM, int WN, int MT, int NT, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void igemm_multi_f32(const IgemmMulti m) {
   int ci = 0;
   while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
-  igemm_body<WM, WN, MT, NT, false, MODE, false>(m.c[ci], (int)blockIdx.x - m.first[ci]);
+  igemm_body<WM, WN, MT, NT, false, MODE, false, false>(m.c[ci], (int)blockIdx.x - m.first[ci]);
+}
+template <int WM, int WN, int MT, int NT, int MODE>
+__global__ __launch_bounds__(kThreads, 3) void igemm_multi_bf16(const IgemmMulti m) {
+  int ci = 0;
+  while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
+  igemm_body<WM, WN, MT, NT, false, MODE, false, true>(m.c[ci], (int)blockIdx.x - m.first[ci]);
 }
 
 // Stream-K second stage: MT*NT blocks per left-over tile, one per 32x32 accumulator tile of
@@ -767,6 +815,10 @@ bool wants_stream_k(long long tiles, int chunks, int groups) {
   return (double)tiles / (double)(rounds * kCUs) < 0.93;
 }
 
+// The bf16 kernels are bound by the address processing of their loads, not by the matrix pipe:
+// smaller tiles fetch more per FLOP and lose there.
+bool bf16_math() { return tt::conv_math() == TT_CONV_MATH_BF16; }
+
 // 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
 // CUs idle or unevenly loaded the reduction is split stream-K fashion; if it is too short for
 // that, 64x64 tiles raise the block count instead.  `small` asks for 64x64 tiles outright: many
@@ -801,9 +853,13 @@ size_t sk_workspace_bytes() { return (size_t)2 * kSkBlocks * 128 * 128 * sizeof(
 
 template <int WM, int WN, int MT, int NT, int MODE, bool AT>
 void launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+  const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
   if (sk_blocks > 0) {
-    igemm_f32<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    if (bf) igemm_bf16<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    else igemm_f32<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     igemm_fixup<WM, WN, MT, NT><<<dim3(p.tiles - p.skDpTiles, MT * NT), kThreads, 0, st>>>(p);
+  } else if (bf) {
+    igemm_bf16<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   } else {
     igemm_f32<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
@@ -883,8 +939,14 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
 template <int WM, int WN, int MT, int NT>
 void launch_multi_config(const IgemmMulti& m, int groups, hipStream_t st) {
   const dim3 grid(m.first[m.n], groups);
-  if (m.c[0].mode == kModeTapMask) igemm_multi_f32<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
-  else igemm_multi_f32<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
+  const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
+  if (m.c[0].mode == kModeTapMask) {
+    if (bf) igemm_multi_bf16<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
+    else igemm_multi_f32<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
+  } else {
+    if (bf) igemm_multi_bf16<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
+    else igemm_multi_f32<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
+  }
 }
 int launch_igemm_multi(IgemmMulti& m, int groups, TileChoice t, int prof_id) {
   tt::ProfScope prof(prof_id);
@@ -975,7 +1037,7 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
   const int M = N * P * Q;
   const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
   const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
-  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ, true, plain && KQ / kBKQ <= 32);
+  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ, true, plain && KQ / kBKQ <= 32 && !bf16_math());
   const int Ipad = ceil_div(Kg, t.bm) * t.bm;
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
@@ -1177,7 +1239,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
       const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
       const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k,
-                                       (plain && KQ / kBKQ <= 32) || !allow_stream_k);
+                                       (plain && KQ / kBKQ <= 32 && !bf16_math()) || !allow_stream_k);
       const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
       KEntry* tab = (KEntry*)((char*)wp + wp_bytes);

@@ -25,6 +25,7 @@ struct State {
   size_t bytes_pooled = 0;
   void* ws = nullptr;
   size_t ws_bytes = 0;
+  int conv_math = TT_CONV_MATH_F32;
   // per-kernel timing
   bool profiling = false;
   std::vector<hipEvent_t> event_pool;
@@ -78,6 +79,7 @@ int fail_hip(hipError_t e, const char* what, const char* file, int line) {
 }
 
 hipStream_t stream() { return S().stream; }
+int conv_math() { return S().conv_math; }
 bool initialised() { return S().ready; }
 
 int workspace(size_t bytes, void** out) {
@@ -270,6 +272,18 @@ int tt_memset(void* dst_dev, int byte_value, size_t bytes) {
   TT_REQUIRE_INIT();
   if (bytes == 0) return 0;
   TT_HIP(hipMemsetAsync(dst_dev, byte_value, bytes, S().stream));
+  return 0;
+}
+
+int tt_set_conv_math(int mode) {
+  TT_REQUIRE(mode == TT_CONV_MATH_F32 || mode == TT_CONV_MATH_BF16, "tt_set_conv_math: unknown mode %d", mode);
+  S().conv_math = mode;
+  return 0;
+}
+
+int tt_get_conv_math(int* mode) {
+  TT_REQUIRE(mode != nullptr, "tt_get_conv_math: null output pointer");
+  *mode = S().conv_math;
   return 0;
 }
 

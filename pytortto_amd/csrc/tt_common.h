@@ -31,6 +31,9 @@ struct ProfScope {
 
 constexpr int kWave = 64;
 
+// Matrix arithmetic of the convolution kernels: TT_CONV_MATH_F32 or TT_CONV_MATH_BF16 (tt_set_conv_math).
+int conv_math();
+
 inline bool fits_i32(long long elems) { return elems >= 0 && elems < 2147483647LL; }
 
 // Unsigned division by a run-time constant without a divide instruction:

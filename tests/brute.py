@@ -146,3 +146,11 @@ def max_pool2d_backward_def(x_shape, grad, arg, accumulate=False):
                     else:
                         dx[nn, cc, where[0], where[1]] = grad[nn, cc, p, q]
     return dx
+
+
+def bf16_round(a):
+    """float32 -> nearest bfloat16 (ties to even), returned as float32: the operand rounding of the
+    optional bf16 convolution variant."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7fff + ((u >> 16) & 1)) & 0xffff0000
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(a))

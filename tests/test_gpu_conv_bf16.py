@@ -1,0 +1,124 @@
+"""GPU checks of the optional bf16 MFMA variant of convolution forward / input gradient.
+
+The reference is float32 throughout, so this variant has no counterpart to be identical to; what
+it computes is pinned exactly instead: both operands rounded to bfloat16 (nearest even), products
+accumulated in float32, bias added in float32.  Products of two bfloat16 values are exact in
+float32, so the oracle run on operands rounded the same way on the host must agree to the
+float32 bar (rtol=1e-4, atol=1e-5 of the tensor's magnitude) -- only the summation order differs.
+Against the oracle on the unrounded operands the stated bound is max|error| <= 1e-2 * max|ref|
+(measured: 2-3e-3).  The weight gradient stays float32 and must not change with the mode.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from tests.brute import bf16_round
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
+from tests.test_gpu_conv import TILE_CASES, CONVT_TILE_CASES
+
+pytestmark = pytest.mark.gpu
+
+LOOSE_BOUND = 1e-2
+
+
+@pytest.fixture
+def bf16_math():
+    from pytortto_amd import _hip
+    _hip.set_conv_math('bf16')
+    try:
+        yield
+    finally:
+        _hip.set_conv_math('f32')
+
+
+def _close(name, got, model, plain):
+    scale = max(1.0, float(np.abs(model).max()))
+    np.testing.assert_allclose(got, model, rtol=1e-4, atol=1e-5 * scale, err_msg=name + ' vs oracle on rounded operands')
+    err = float(np.abs(got - plain).max()) / (float(np.abs(plain).max()) or 1.0)
+    assert err <= LOOSE_BOUND, f'{name}: {err:.3g} of max|ref| against the float32 oracle'
+
+
+@pytest.mark.parametrize('case', CONV_CASES + TILE_CASES + random_conv_cases(40, 123))
+def test_conv_bf16_forward_and_input_gradient(case, bf16_math):
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((n, c, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((k, c // g, r, s)) / np.sqrt(c // g * r * s)).astype(np.float32)
+    b = rng.standard_normal(k).astype(np.float32)
+    y32, xpad = oracle.convolution_forward(x, w, b, st, pd, dl, g)
+    gy = rng.standard_normal(y32.shape).astype(np.float32)
+    dx32 = oracle.conv2d_backward_x(gy, w, st, pd, dl, g, x_hw=(h, w_))
+    xr, wr, gyr = bf16_round(x), bf16_round(w), bf16_round(gy)
+    y_model = oracle.convolution_forward(xr.astype(np.float64), wr.astype(np.float64), b.astype(np.float64), st, pd, dl, g)[0]
+    dx_model = oracle.conv2d_backward_x(gyr.astype(np.float64), wr.astype(np.float64), st, pd, dl, g, x_hw=(h, w_))
+
+    xd, wd, gyd = hiparray(x), hiparray(w), hiparray(gy)
+    y = ops.conv2d_fwd(xd, wd, hiparray(b), st, pd, dl, g).get()
+    dx = ops.conv2d_dgrad(gyd, wd, None, (h, w_), st, pd, dl, g).get()
+    _close('y', y, y_model, y32)
+    _close('dx', dx, dx_model, dx32)
+
+
+@pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES + random_convt_cases(12, 321))
+def test_conv_transpose_bf16_forward_and_input_gradient(case, bf16_math):
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    n, ci, h, w_, co, r, s, st, pd, op, dl, g = case
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((n, ci, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((ci, co // g, r, s)) / np.sqrt(ci // g * r * s)).astype(np.float32)
+    b = rng.standard_normal(co).astype(np.float32)
+    y32 = oracle.transposed_convolution_forward(x, w, b, st, pd, op, dl, g)
+    gy = rng.standard_normal(y32.shape).astype(np.float32)
+    dx32 = oracle.transposed_convolution_backward(gy, x, w, st, pd, dl, g)[0]
+    xr, wr, gyr = (bf16_round(a).astype(np.float64) for a in (x, w, gy))
+    y_model = oracle.transposed_convolution_forward(xr, wr, b.astype(np.float64), st, pd, op, dl, g)
+    dx_model = oracle.transposed_convolution_backward(gyr, xr, wr, st, pd, dl, g)[0]
+
+    xd, wd, gyd = hiparray(x), hiparray(w), hiparray(gy)
+    y = ops.conv2d_dgrad(xd, wd, hiparray(b), y32.shape[-2:], st, pd, dl, g).get()
+    dx = ops.conv2d_fwd(gyd, wd, None, st, pd, dl, g).get()
+    _close('y', y, y_model, y32)
+    _close('dx', dx, dx_model, dx32)
+
+
+def test_weight_gradient_and_other_ops_do_not_depend_on_the_mode():
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(6)
+    x = hiparray(rng.standard_normal((8, 32, 14, 14), dtype=np.float32))
+    gy = hiparray(rng.standard_normal((8, 48, 14, 14), dtype=np.float32))
+    w = hiparray(rng.standard_normal((48, 32, 3, 3), dtype=np.float32))
+    args = ((1, 1), (1, 1), (1, 1), 1)
+    assert _hip.get_conv_math() == 'f32'
+    dw = ops.conv2d_wgrad(x, gy, (48, 32, 3, 3), *args).get()
+    y = ops.conv2d_fwd(x, w, None, *args).get()
+    _hip.set_conv_math('bf16')
+    try:
+        assert _hip.get_conv_math() == 'bf16'
+        np.testing.assert_array_equal(ops.conv2d_wgrad(x, gy, (48, 32, 3, 3), *args).get(), dw)
+        y_bf = ops.conv2d_fwd(x, w, None, *args).get()
+        assert np.abs(y_bf - y).max() > 0          # the mode is really in effect
+    finally:
+        _hip.set_conv_math('f32')
+    np.testing.assert_array_equal(ops.conv2d_fwd(x, w, None, *args).get(), y)   # and really off again
+    with pytest.raises(ValueError):
+        _hip.set_conv_math('fp8')
+
+
+def test_module_api_switch():
+    import pytortto_amd as tt
+    tt.manual_seed(0)
+    conv = tt.nn.Conv2d(16, 32, 3, padding=1).cuda()
+    x = tt.randn(4, 16, 12, 12).cuda()
+    y = conv(x).data.get()
+    tt.cuda.set_conv_math('bf16')
+    try:
+        assert tt.cuda.get_conv_math() == 'bf16'
+        y_bf = conv(x).data.get()
+    finally:
+        tt.cuda.set_conv_math('f32')
+    err = np.abs(y_bf - y).max() / np.abs(y).max()
+    assert 0 < err <= LOOSE_BOUND
