@@ -815,8 +815,8 @@ bool wants_stream_k(long long tiles, int chunks, int groups) {
   return (double)tiles / (double)(rounds * kCUs) < 0.93;
 }
 
-// The bf16 kernels are bound by the address processing of their loads, not by the matrix pipe:
-// smaller tiles fetch more per FLOP and lose there.
+// The bf16 kernels are bound by their fetch path, not by the matrix pipe: smaller tiles fetch more
+// per FLOP and lose there.
 bool bf16_math() { return tt::conv_math() == TT_CONV_MATH_BF16; }
 
 // 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
