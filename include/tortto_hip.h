@@ -82,14 +82,16 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
 
 /* ---- convolution ------------------------------------------------------------------------- */
 
-/* Matrix arithmetic of tt_conv2d_fwd_f32 and tt_conv2d_dgrad_f32 (no counterpart in the reference,
+/* Matrix arithmetic of the three convolution passes (no counterpart in the reference,
  * whose path is float32 throughout).  TT_CONV_MATH_F32 (the default) multiplies in float32 on
  * v_mfma_f32_32x32x2_f32 and is the mode that meets the reference's tolerances.
  * TT_CONV_MATH_BF16 is the optional reduced-precision variant: tensors stay float32 in memory,
  * both operands are rounded to bfloat16 (nearest even) on their way into
- * v_mfma_f32_32x32x16_bf16 and products are accumulated in float32; results differ from the
- * float32 ones by about 2^-8 of the operands' magnitude per term.  The weight gradient is
- * computed in float32 in both modes.  The setting is process-wide and applies to later calls. */
+ * v_mfma_f32_32x32x16_bf16 and products are accumulated in float32 (the weight gradient's
+ * partial sums are still combined in float64); results differ from the float32 ones by about
+ * 2^-8 of the operands' magnitude per term.  It applies to tt_conv2d_fwd_f32,
+ * tt_conv2d_dgrad_f32 and tt_conv2d_wgrad_f32.  The setting is process-wide and applies to
+ * later calls. */
 enum { TT_CONV_MATH_F32 = 0, TT_CONV_MATH_BF16 = 1 };
 int tt_set_conv_math(int mode);
 int tt_get_conv_math(int* mode);   /* host pointer */

@@ -38,8 +38,8 @@ class cuda:
 
     @staticmethod
     def set_conv_math(mode):
-        """Not in the reference (float32 throughout): ``'f32'`` (default) or ``'bf16'`` -- convolution
-        forward / input gradient with operands rounded to bfloat16 inside the kernel and float32
+        """Not in the reference (float32 throughout): ``'f32'`` (default) or ``'bf16'`` -- the three
+        convolution passes with operands rounded to bfloat16 inside the kernels and float32
         accumulation.  Tensors stay float32; results then differ from the float32 path by a few 1e-3
         of their magnitude."""
         _hip.set_conv_math(mode)

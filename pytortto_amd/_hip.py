@@ -169,7 +169,7 @@ CONV_MATH = {'f32': 0, 'bf16': 1}
 
 
 def set_conv_math(mode):
-    """Matrix arithmetic of convolution forward / input gradient: 'f32' (default, the mode that meets
+    """Matrix arithmetic of the three convolution passes: 'f32' (default, the mode that meets
     the reference's tolerances) or 'bf16' (operands rounded to bfloat16 inside the kernel, float32
     accumulation; tensors stay float32)."""
     if mode not in CONV_MATH:

@@ -28,6 +28,7 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
 constexpr int kBK = 32;        // pixels per chunk
@@ -98,8 +99,10 @@ __global__ void wgrad_build_pixtab(int4* __restrict__ tab, Wgrad p, int entries,
 // (thread = (row group of 32, pixel quad) instead of (row group of 8, pixel)).  VA needs P*Q to be
 // a multiple of 4 so that a quad never straddles two images, VB in addition a 1x1, stride-1,
 // unpadded layer, where x is indexed by the output pixel like dy and has no padding to mask.
-template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
-__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_f32(const Wgrad p) {
+// BF: the optional bf16 variant (tt_set_conv_math): operands rounded to bfloat16 after the LDS
+// read, v_mfma_f32_32x32x16_bf16, float32 accumulation.
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB, bool BF>
+__device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   static_assert(WM * WN == 4, "four waves per block");
   static_assert(BUF || (!VA && !VB), "vector fetches belong to the buffer path");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
@@ -310,6 +313,45 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
   constexpr int kStore = 5 * T / 8, kSync = T - 4;
   constexpr int SPS = (L + (kSync - kStore) - 1) / (kSync - kStore);   // LDS writes per slot
   auto chunk_body = [&](const int buf, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
+    if constexpr (BF) {
+      // Two bf16 MFMAs per accumulator contract the chunk's 32 pixels (a lane's eight k values of
+      // each are pixels 16*half + 4*h .. +3 and 16*half + 8 + 4*h .. +3, the same for both
+      // operands): a sixteenth of the fp32 matrix time, nothing to weave the loads into.
+      decompose(nchunk, nnchunk);
+#pragma unroll
+      for (int li = 0; li < L; ++li) load_step(li);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (half == 1) read_ops(0, buf, 2);
+        read_ops(1, buf, 2 * half + 1);
+        bf16x8 a[MT], b[NT];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int xx = 0; xx < MT; ++xx) {
+            a[xx][j] = (__bf16)opA[0][xx][j];
+            a[xx][4 + j] = (__bf16)opA[1][xx][j];
+          }
+#pragma unroll
+          for (int yy = 0; yy < NT; ++yy) {
+            b[yy][j] = (__bf16)opB[0][yy][j];
+            b[yy][4 + j] = (__bf16)opB[1][yy][j];
+          }
+        }
+#pragma unroll
+        for (int xx = 0; xx < MT; ++xx)
+#pragma unroll
+          for (int yy = 0; yy < NT; ++yy)
+            acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[xx], b[yy], acc[xx][yy], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int li = 0; li < L; ++li) store_step(buf ^ 1, li);
+      __syncthreads();
+      read_ops(0, buf ^ 1, 0);
+      return;
+    }
 #pragma unroll
     for (int s = 0; s < T; ++s) {
       const int kk = s / PK, rem = s % PK;
@@ -374,6 +416,15 @@ __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 
         if (i < p.Kg) out[(size_t)i * p.J + j] = acc[xx][yy][r];
       }
   }
+}
+
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
+__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_f32(const Wgrad p) {
+  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, false>(p);
+}
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
+__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_bf16(const Wgrad p) {
+  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, true>(p);
 }
 
 // dw[e] = sum over splits of partial[s][e] in float64.  A block covers 64 float4 columns with
@@ -458,6 +509,13 @@ int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
 
 template <int WM, int WN, int MT, int NT>
 void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStream_t st) {
+  if (tt::conv_math() == TT_CONV_MATH_BF16) {
+    if (buf && va && vb) wgrad_bf16<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
+    else if (buf && va) wgrad_bf16<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
+    else if (buf) wgrad_bf16<WM, WN, MT, NT, true, false, false><<<grid, kThreads, 0, st>>>(p);
+    else wgrad_bf16<WM, WN, MT, NT, false, false, false><<<grid, kThreads, 0, st>>>(p);
+    return;
+  }
   if (buf && va && vb) wgrad_f32<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
   else if (buf && va) wgrad_f32<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
   else if (buf) wgrad_f32<WM, WN, MT, NT, true, false, false><<<grid, kThreads, 0, st>>>(p);
