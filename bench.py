@@ -423,6 +423,14 @@ def main():
                  'loss_first_last': [round(m_losses[0], 4), round(m_losses[-1], 4)],
                  'note': 'wall clock around the Python loop, launches asynchronous; fp32, synthetic 3x224x224 input'}
         call('tt_empty_cache')
+        _hip.set_conv_math('bf16')   # the optional variant, reported beside the fp32 figure
+        try:
+            b_ips, b_ms, b_wall, b_losses = resnet50_train_step(_hip, max(3, args.steps // 2), 2)
+        finally:
+            _hip.set_conv_math('f32')
+        model['with_bf16_conv_math'] = {'value': round(b_ips, 1), 'unit': 'images/s', 'ms_per_step': round(b_wall, 2),
+                                        'loss_first_last': [round(b_losses[0], 4), round(b_losses[-1], 4)]}
+        call('tt_empty_cache')
 
     # ---- what the device sustains on the two bounding resources, measured in this run ----------
     mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
