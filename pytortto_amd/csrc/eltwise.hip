@@ -31,18 +31,29 @@ __global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a,
   // results that are not accumulated in place stream out past the caches
   constexpr bool kStreamOut = OP == kRelu || OP == kReluBwd || OP == kAdd || OP == kLeakyRelu || OP == kLeakyReluBwd;
   constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy || OP == kLeakyReluBwd;
+  // two-input kernels whose inputs are read for the last time here (a gradient and the saved
+  // activation, the two branches of a residual add) stream them in past the caches too: 8-9 %
+  // faster than allocating loads at 200 MB per tensor; one-input kernels are faster with plain loads
+  constexpr bool kStreamIn = kStreamOut && kUseB;
   const size_t n4 = n >> 2;
   const size_t stride = (size_t)gridDim.x * kThreads;
   for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n4; i += stride) {
     float4 va = make_float4(0.f, 0.f, 0.f, 0.f), vb = va, o;
-    if (kUseA) va = reinterpret_cast<const float4*>(a)[i];
-    if (kUseB) vb = reinterpret_cast<const float4*>(b)[i];
+    typedef float fx4 __attribute__((ext_vector_type(4)));
+    if (kUseA) {
+      // (the increment of a gradient accumulation is read for the last time as well)
+      if (kStreamIn || OP == kAxpy) { const fx4 t = __builtin_nontemporal_load(reinterpret_cast<const fx4*>(a) + i); va = make_float4(t.x, t.y, t.z, t.w); }
+      else va = reinterpret_cast<const float4*>(a)[i];
+    }
+    if (kUseB) {
+      if (kStreamIn) { const fx4 t = __builtin_nontemporal_load(reinterpret_cast<const fx4*>(b) + i); vb = make_float4(t.x, t.y, t.z, t.w); }
+      else vb = reinterpret_cast<const float4*>(b)[i];
+    }
     o.x = apply1<OP>(va.x, vb.x, alpha);
     o.y = apply1<OP>(va.y, vb.y, alpha);
     o.z = apply1<OP>(va.z, vb.z, alpha);
     o.w = apply1<OP>(va.w, vb.w, alpha);
     if (kStreamOut) {
-      typedef float fx4 __attribute__((ext_vector_type(4)));
       const fx4 ov = {o.x, o.y, o.z, o.w};
       __builtin_nontemporal_store(ov, reinterpret_cast<fx4*>(out) + i);
     } else {
