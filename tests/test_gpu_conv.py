@@ -106,6 +106,12 @@ def test_conv_without_bias():
     _run_conv((2, 4, 8, 8, 6, 3, 3, (1, 1), (1, 1), (1, 1), 1), bias=False)
 
 
+@pytest.mark.parametrize('case', TILE_CASES + random_conv_cases(24, 77))
+def test_conv_tile_configurations_without_bias(case):
+    """Without a bias the stores take the scalar-addressed path when the row count is a multiple of 8."""
+    _run_conv(case, seed=5, bias=False)
+
+
 CONVT_TILE_CASES = [
     (16, 100, 1, 1, 512, 4, 4, (1, 1), (0, 0), (0, 0), (1, 1), 1),   # DCGAN layer 1 (reduced batch)
     (8, 256, 8, 8, 128, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),    # DCGAN upsampling layer
