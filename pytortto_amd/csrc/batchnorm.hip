@@ -479,9 +479,129 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) 
   if (kMode == 2) sweep2_flat<true, 1>(a.x, a.dy, a.dx, g, c, split, k);
 }
 
+// ---- small channels: one kernel per pass ---------------------------------------------------------
+// When a channel's N*HW values fit the registers of one block (<= kThreads * EMAX), the block
+// reads them once, reduces, and applies from registers: S read + S written forward, 2S + S
+// backward instead of 3S and 5S, and one launch instead of two.  Grid = C blocks; g.hwv_div
+// divides by HW.  The deep layers of a network (7x7 to 16x16 planes, hundreds of channels) are
+// of this kind.  Statistics and coefficients follow the two-sweep kernels' formulas exactly.
+
+template <int EMAX, typename F>
+__device__ __forceinline__ void for_channel_elements(const Geometry& g, F&& f) {
+  const int total = g.N * g.HW;
+  const size_t image = (size_t)g.C * g.HW;
+#pragma unroll
+  for (int k = 0; k < EMAX; ++k) {
+    const int e = (int)threadIdx.x + k * kThreads;
+    if (e < total) {
+      const uint32_t n = tt::fd_div((uint32_t)e, g.hwv_div);
+      f(k, (size_t)n * image + ((uint32_t)e - n * (uint32_t)g.HW));
+    }
+  }
+}
+
+template <int EMAX>
+__global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) {
+  __shared__ double red[2 * kWaves];
+  __shared__ Coef sk;
+  const int c = blockIdx.x;
+  const float* __restrict__ xc = a.x + (size_t)c * g.HW;
+  float* __restrict__ yc = a.y + (size_t)c * g.HW;
+  const float shift = xc[0];
+  float v[EMAX];
+  for_channel_elements<EMAX>(g, [&](int k, size_t off) { v[k] = xc[off]; });
+  double s1 = 0.0, s2 = 0.0;
+  for_channel_elements<EMAX>(g, [&](int k, size_t) {
+    const double d = (double)(v[k] - shift);
+    s1 += d;
+    s2 += d * d;
+  });
+  block_sum2(s1, s2, red);
+  if (threadIdx.x == 0) {
+    const double m = (double)g.N * (double)g.HW;
+    const double d1 = s1 / m;
+    const float mean = (float)((double)shift + d1);
+    const float var = (float)fmax(s2 / m - d1 * d1, 0.0);
+    const float var_eps = __fadd_rn(var, a.eps);
+    const float sd = __fsqrt_rn(var_eps);
+    sk.m = mean;
+    sk.k1 = __fdiv_rn(a.gamma ? a.gamma[c] : 1.0f, sd);
+    sk.k0 = a.beta ? a.beta[c] : 0.0f;
+    sk.k2 = 0.f;
+    a.save_mean[c] = mean;
+    a.save_var_eps[c] = var_eps;
+    a.save_sd[c] = sd;
+    if (a.rm_in) {   // separate roundings, as NumPy evaluates (1-m)*rm + m*mean on float32 arrays
+      a.rm_out[c] = __fadd_rn(__fmul_rn(a.one_minus_mom, a.rm_in[c]), __fmul_rn(a.mom, mean));
+      a.rv_out[c] = __fadd_rn(__fmul_rn(a.one_minus_mom, a.rv_in[c]), __fmul_rn(a.mom, __fmul_rn(var, a.unbias)));
+    }
+  }
+  __syncthreads();
+  const Coef k = sk;
+  for_channel_elements<EMAX>(g, [&](int kk, size_t off) {
+    __builtin_nontemporal_store(fmaf(v[kk] - k.m, k.k1, k.k0), yc + off);
+  });
+}
+
+template <int EMAX>
+__global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) {
+  __shared__ double red[2 * kWaves];
+  __shared__ Coef sk;
+  const int c = blockIdx.x;
+  const float* __restrict__ xc = a.x + (size_t)c * g.HW;
+  const float* __restrict__ dyc = a.dy + (size_t)c * g.HW;
+  const float mean = a.save_mean[c];
+  float v[EMAX], gq[EMAX];
+  for_channel_elements<EMAX>(g, [&](int k, size_t off) {
+    v[k] = __builtin_nontemporal_load(xc + off);
+    gq[k] = __builtin_nontemporal_load(dyc + off);
+  });
+  double s_dy = 0.0, s_dyxmu = 0.0;
+  for_channel_elements<EMAX>(g, [&](int k, size_t) {
+    s_dy += (double)gq[k];
+    s_dyxmu += (double)gq[k] * (double)(v[k] - mean);
+  });
+  block_sum2(s_dy, s_dyxmu, red);
+  if (threadIdx.x == 0) {
+    const double m = (double)g.N * (double)g.HW;
+    const double sd = (double)a.save_sd[c];
+    const double var_eps = (double)a.save_var_eps[c];
+    const double k1 = (a.gamma ? (double)a.gamma[c] : 1.0) / sd;
+    sk.m = mean;
+    sk.k1 = (float)k1;
+    sk.k0 = (float)(-k1 * s_dy / m);
+    sk.k2 = (float)(-k1 * s_dyxmu / (m * var_eps));
+    if (a.dbeta) a.dbeta[c] = (float)s_dy;
+    if (a.dgamma) a.dgamma[c] = (float)(s_dyxmu / sd);
+  }
+  if (a.dx == nullptr) return;
+  __syncthreads();
+  const Coef k = sk;
+  float* __restrict__ dxc = a.dx + (size_t)c * g.HW;
+  for_channel_elements<EMAX>(g, [&](int kk, size_t off) {
+    __builtin_nontemporal_store(fmaf(gq[kk], k.k1, fmaf(v[kk] - k.m, k.k2, k.k0)), dxc + off);
+  });
+}
+
 // ---- host side -------------------------------------------------------------------------------------
 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// Channels small enough for the single-kernel passes, and enough of them to fill the device.
+constexpr int kSmallMax = 64;   // values per thread
+int small_channel_capacity(int N, int C, int HW) {
+  const long long total = (long long)N * HW;
+  if (C < 128 || total > (long long)kThreads * kSmallMax) return 0;
+  return total <= (long long)kThreads * 16 ? 16 : kSmallMax;
+}
+Geometry small_geometry(int N, int C, int HW) {
+  Geometry g{};
+  g.N = N; g.C = C; g.HW = HW;
+  g.splits = 1;
+  g.per_block = 0;
+  g.hwv_div = tt::make_fastdiv((uint32_t)HW);
+  return g;
+}
 
 // Picks the kernel flavour and how a channel is shared between blocks.
 constexpr int kStreamBatches = 4;
@@ -571,6 +691,25 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   const bool track = running_mean_in && running_var_in;
   TT_REQUIRE(!track || (running_mean_out && running_var_out),
              "tt_bn_fwd_train_f32: running statistics given without output buffers");
+  FwdArgs a{};
+  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
+  a.save_mean = save_mean; a.save_var_eps = save_var_eps; a.save_sd = save_sd;
+  a.rm_in = track ? running_mean_in : nullptr; a.rv_in = track ? running_var_in : nullptr;
+  a.rm_out = running_mean_out; a.rv_out = running_var_out;
+  a.given_mean = nullptr; a.given_var = nullptr;
+  a.one_minus_mom = (float)(1.0 - momentum);
+  a.mom = (float)momentum;
+  a.unbias = (float)((double)m / (double)(m - 1));
+  a.eps = (float)eps;
+  hipStream_t st = tt::stream();
+  if (const int cap = small_channel_capacity(N, C, HW)) {
+    tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
+    const Geometry gs = small_geometry(N, C, HW);
+    if (cap == 16) bn_fwd_small<16><<<C, kThreads, 0, st>>>(a, gs);
+    else bn_fwd_small<kSmallMax><<<C, kThreads, 0, st>>>(a, gs);
+    TT_LAUNCH_CHECK();
+    return 0;
+  }
   Geometry g, gr;
   int mode, rmode;
   plan(N, C, HW, &g, &mode);
@@ -583,19 +722,8 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
     launch_reduce<0>(rmode, dim3(gr.splits, C), x, x, nullptr, (double2*)ws, gr);
   }
   TT_LAUNCH_CHECK();
-  FwdArgs a{};
-  a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
-  a.save_mean = save_mean; a.save_var_eps = save_var_eps; a.save_sd = save_sd;
-  a.rm_in = track ? running_mean_in : nullptr; a.rv_in = track ? running_var_in : nullptr;
-  a.rm_out = running_mean_out; a.rv_out = running_var_out;
-  a.given_mean = nullptr; a.given_var = nullptr;
   a.partial = (const double2*)ws;
   a.partial_splits = gr.splits;
-  a.one_minus_mom = (float)(1.0 - momentum);
-  a.mom = (float)momentum;
-  a.unbias = (float)((double)m / (double)(m - 1));
-  a.eps = (float)eps;
-  hipStream_t st = tt::stream();
   {
     tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
     if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
@@ -640,6 +768,15 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const flo
   if (check_shape("tt_bn_bwd_f32", N, C, HW)) return -1;
   TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "tt_bn_bwd_f32: null tensor pointer");
   if (!dx && !dgamma && !dbeta) return 0;
+  if (const int cap = small_channel_capacity(N, C, HW)) {
+    tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
+    const Geometry gs = small_geometry(N, C, HW);
+    BwdArgs b{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, nullptr, 0};
+    if (cap == 16) bn_bwd_small<16><<<C, kThreads, 0, tt::stream()>>>(b, gs);
+    else bn_bwd_small<kSmallMax><<<C, kThreads, 0, tt::stream()>>>(b, gs);
+    TT_LAUNCH_CHECK();
+    return 0;
+  }
   Geometry g, gr;
   int mode, rmode;
   plan(N, C, HW, &g, &mode);
@@ -685,6 +822,10 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
 int tt_workspace_size_bn_f32(size_t* bytes, int N, int C, int HW) {
   TT_REQUIRE(bytes, "tt_workspace_size_bn_f32: null result pointer");
   if (check_shape("tt_workspace_size_bn_f32", N, C, HW)) return -1;
+  if (small_channel_capacity(N, C, HW)) {   // single-kernel passes: no partials
+    *bytes = 0;
+    return 0;
+  }
   Geometry gr;
   int rmode;
   plan_reduce(N, C, HW, &gr, &rmode);
