@@ -213,3 +213,64 @@ def _random_bn_shapes(count, seed):
 @pytest.mark.parametrize('shape', _random_bn_shapes(40, 31), ids=lambda s: '%dx%dx%dx%d' % s)
 def test_bn_random_shapes(shape):
     test_bn_train_fwd_bwd_matches_oracle(shape)
+
+
+# at least 128 channels of at most 16384 values each: the single-kernel passes (one block per channel
+# keeps the channel in registers); the last two sit just inside and just outside that limit
+SMALL_CHANNEL_SHAPES = [
+    (64, 256, 7, 7),      # 3136 values: 16 per thread
+    (32, 128, 14, 14),    # 6272 values: 64-per-thread instance, partly filled
+    (2, 128, 1, 1),       # two values per channel
+    (3, 200, 5, 7),       # odd plane, threads without a value
+    (128, 512, 4, 4),     # DCGAN / PreAct-ResNet-18 deepest layers
+    (16, 130, 31, 33),    # 16368 values
+    (64, 128, 16, 16),    # 16384 values: exactly the capacity
+    (65, 128, 16, 16),    # 16640 values: back on the two-sweep kernels
+]
+
+
+@pytest.mark.parametrize('shape', SMALL_CHANNEL_SHAPES, ids=lambda s: '%dx%dx%dx%d' % s)
+def test_bn_small_channels_single_kernel(shape):
+    test_bn_train_fwd_bwd_matches_oracle(shape)
+
+
+def test_bn_small_channels_optional_arguments_and_stability():
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    shape = (16, 160, 9, 9)
+    x, gamma, beta, dy = _inputs(shape, seed=8)
+    # no affine parameters, no running statistics, only dx wanted
+    y_ref, saved, _, _ = oracle.batch_norm_forward(x, None, None, None, None, True, 0.1, 1e-5)
+    dx_ref, _, _ = oracle.batch_norm_backward(dy, x, None, saved, need=(True, False, False))
+    xd, dyd = hiparray(x), hiparray(dy)
+    y, mean, var_eps, sd, rm, rv = ops.bn_fwd_train(xd, None, None, None, None, 0.1, 1e-5)
+    assert rm is None and rv is None
+    dx, dg, db = ops.bn_bwd(xd, dyd, None, mean, var_eps, sd, need=(True, False, False))
+    assert dg is None and db is None
+    _close(y.get(), y_ref)
+    _close(dx.get(), dx_ref, rtol=1e-4, atol_scale=1e-5)
+    # only the parameter gradients wanted
+    gd = hiparray(gamma)
+    y_ref, saved, _, _ = oracle.batch_norm_forward(x, gamma, beta, None, None, True, 0.1, 1e-5)
+    _, dg_ref, db_ref = oracle.batch_norm_backward(dy, x, gamma, saved)
+    _, mean, var_eps, sd, _, _ = ops.bn_fwd_train(xd, gd, hiparray(beta), None, None, 0.1, 1e-5)
+    dx, dg, db = ops.bn_bwd(xd, dyd, gd, mean, var_eps, sd, need=(False, True, True))
+    assert dx is None
+    _close(dg.get(), dg_ref, rtol=1e-4, atol_scale=1e-5)
+    _close(db.get(), db_ref, rtol=1e-4, atol_scale=1e-5)
+    # |mean| >> sigma
+    np.random.seed(9)
+    xs = (1000 + 0.5 * np.random.randn(8, 128, 12, 12)).astype(np.float32)
+    _, mean, var_eps, _, _, _ = ops.bn_fwd_train(hiparray(xs), None, None, None, None, 0.1, 0.0)
+    np.testing.assert_allclose(var_eps.get(), xs.astype(np.float64).var((0, 2, 3)), rtol=1e-4)
+    np.testing.assert_allclose(mean.get(), xs.astype(np.float64).mean((0, 2, 3)), rtol=1e-6)
+    # running statistics over three steps
+    c = 144
+    rm, rv = np.zeros(c, np.float32), np.ones(c, np.float32)
+    rmd, rvd = hiparray(rm), hiparray(rv)
+    for step in range(3):
+        x, gamma, beta, _ = _inputs((6, c, 10, 10), seed=20 + step)
+        _, _, rm, rv = oracle.batch_norm_forward(x, gamma, beta, rm, rv, True, 0.3, 1e-5)
+        _, _, _, _, rmd, rvd = ops.bn_fwd_train(hiparray(x), hiparray(gamma), hiparray(beta), rmd, rvd, 0.3, 1e-5)
+    _close(rmd.get(), rm)
+    _close(rvd.get(), rv)
