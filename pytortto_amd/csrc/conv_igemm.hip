@@ -331,20 +331,14 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
     const int soff = 4 * (chunk * (4 * kBKQ) + j) * p.kStride;
     greg[j] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(srcSrd, bvoff, soff, 0));
   };
+  // In this mode the gathered tile lies in LDS as it lies in memory, [k][pixel]: a fetched
+  // 16-byte vector is written as it is (consecutive lanes, consecutive addresses: no bank
+  // conflicts, where scattering its four pixels into the k-quad layout cost up to eight-way
+  // ones), and read_ops picks a lane's four k values with four dword reads off one address.
   auto store_g = [&](int buf) __attribute__((always_inline)) {
-    // transpose in registers: pixel e of the quad gets this thread's GR consecutive k values
+    float* tile = reinterpret_cast<float*>(&Bs[buf][0][0]);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float* dst = reinterpret_cast<float*>(&Bs[buf][gkr >> 2][4 * gpq + e]) + (gkr & 3);
-      if constexpr (GR == 4) {
-        *reinterpret_cast<floatx4*>(dst) = floatx4{greg[0][e], greg[1][e], greg[2][e], greg[3][e]};
-      } else if constexpr (GR == 2) {
-        typedef float floatx2 __attribute__((ext_vector_type(2)));
-        *reinterpret_cast<floatx2*>(dst) = floatx2{greg[0][e], greg[1][e]};
-      } else {
-        *dst = greg[0][e];
-      }
-    }
+    for (int j = 0; j < GR; ++j) *reinterpret_cast<floatx4*>(tile + (gkr + j) * BN + 4 * gpq) = greg[j];
   };
 
   floatx4 areg[A_ITEMS];
@@ -420,7 +414,15 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
 #pragma unroll
       for (int x = 0; x < MT; ++x) opA[set][kk][x] = As[buf][kk * 2 + h][(wm * MT + x) * 32 + l32];
 #pragma unroll
-      for (int y = 0; y < NT; ++y) opB[set][kk][y] = Bs[buf][kk * 2 + h][(wn * NT + y) * 32 + l32];
+      for (int y = 0; y < NT; ++y) {
+        if constexpr (GEMM) {
+          const float* tile = reinterpret_cast<const float*>(&Bs[buf][0][0]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) opB[set][kk][y][j] = tile[(4 * (kk * 2 + h) + j) * BN + (wn * NT + y) * 32 + l32];
+        } else {
+          opB[set][kk][y] = Bs[buf][kk * 2 + h][(wn * NT + y) * 32 + l32];
+        }
+      }
     }
   };
 
