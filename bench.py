@@ -48,7 +48,7 @@ BATCH = 64
 # x1.0).  Counters cannot be read from inside this script, so the figures of the last counter
 # run are carried here; the summary with the commands is in the profiles directory
 # (bench_hbm_traffic_fetch_write_size.txt).
-IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 209.5e6      # igemm_f32 + igemm_multi_f32 + igemm_fixup, mean over the 106 launches of a step (106.9e6 algorithmic)
+IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 209.6e6      # igemm_f32 + igemm_multi_f32 + igemm_fixup, mean over the 106 launches of a step (106.9e6 algorithmic)
 BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.3e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
 MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH = 314.6e6    # dy + taps read, dx written (308.3e6 algorithmic)
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
