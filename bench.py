@@ -208,6 +208,77 @@ def resnet50_train_step(hip, steps, warmup, batch=BATCH):
     return batch / (wall * 1e-3), ms, wall, losses
 
 
+def preact18_stack_step(hip, steps, warmup, batch=128):
+    """Forward + backward of the PreAct-ResNet-18 basic-block stack of the reference's
+    examples/resnet/preact_resnet18 notebook at batch 128, 3x32x32, through the module API: conv3x3
+    3->64, stages (64, 128, 256, 512) of two blocks, block = BN-ReLU -> [conv3x3(stride) - BN - ReLU -
+    conv3x3] + shortcut (identity, or conv1x1 stride 2 on the block input), no biases, BatchNorm in
+    training mode, upstream gradient on the last stage's output.  Returns (ms per step, wall ms)."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    F = nn.functional
+
+    class Block(nn.Module):
+        def __init__(self, cin, cout, stride):
+            super().__init__()
+            self.bn1, self.conv1 = nn.BatchNorm2d(cin), nn.Conv2d(cin, cout, 3, stride, 1, bias=False)
+            self.bn2, self.conv2 = nn.BatchNorm2d(cout), nn.Conv2d(cout, cout, 3, 1, 1, bias=False)
+            self.shortcut = None if stride == 1 and cin == cout else nn.Conv2d(cin, cout, 1, stride, bias=False)
+
+        def forward(self, x):
+            out = self.conv1(F.relu(self.bn1(x)))
+            out = self.conv2(F.relu(self.bn2(out)))
+            return out + (x if self.shortcut is None else self.shortcut(x))
+
+    tt.manual_seed(0)
+    layers, cin = [nn.Conv2d(3, 64, 3, 1, 1, bias=False)], 64
+    for cout, stride in ((64, 1), (128, 2), (256, 2), (512, 2)):
+        layers += [Block(cin, cout, stride), Block(cout, cout, 1)]
+        cin = cout
+    net = nn.Sequential(*layers)
+    net.cuda()
+    rng = np.random.default_rng(0)
+    x = tt.tensor(rng.standard_normal((batch, 3, 32, 32), dtype=np.float32)).cuda()
+    g = tt.tensor(rng.standard_normal((batch, 512, 4, 4), dtype=np.float32)).cuda()
+
+    def step():
+        for q in net.parameters():
+            q.grad = None
+        net(x).backward(g)
+
+    ms, wall = timed_steps(hip, step, steps, warmup)
+    del net, x, g
+    return ms, wall
+
+
+def dcgan_generator_step(hip, steps, warmup, batch=128):
+    """Forward + backward of the DCGAN-style generator: latent [batch,100,1,1] -> ConvTranspose2d
+    4x4 stride 1 to 512 channels, then 4x4 / stride 2 / padding 1 to 256, 128, 64 and 3 channels
+    (64x64), BatchNorm2d + ReLU between, no biases.  Returns (ms per step, wall ms)."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    tt.manual_seed(0)
+    layers, cin = [], 100
+    for cout, stride, pad in ((512, 1, 0), (256, 2, 1), (128, 2, 1), (64, 2, 1)):
+        layers += [nn.ConvTranspose2d(cin, cout, 4, stride, pad, bias=False), nn.BatchNorm2d(cout), nn.ReLU()]
+        cin = cout
+    layers.append(nn.ConvTranspose2d(cin, 3, 4, 2, 1, bias=False))
+    net = nn.Sequential(*layers)
+    net.cuda()
+    rng = np.random.default_rng(0)
+    z = tt.tensor(rng.standard_normal((batch, 100, 1, 1), dtype=np.float32)).cuda()
+    g = tt.tensor(rng.standard_normal((batch, 3, 64, 64), dtype=np.float32)).cuda()
+
+    def step():
+        for q in net.parameters():
+            q.grad = None
+        net(z).backward(g)
+
+    ms, wall = timed_steps(hip, step, steps, warmup)
+    del net, z, g
+    return ms, wall
+
+
 def cpu_baseline_pool(batch):
     """(bytes counted, seconds) of the oracle's MaxPool2d forward + backward."""
     import oracle
@@ -432,6 +503,29 @@ def main():
                                         'loss_first_last': [round(b_losses[0], 4), round(b_losses[-1], 4)]}
         call('tt_empty_cache')
 
+    # ---- the other two stack configurations, through the module API -----------------------------
+    stacks = None
+    if not args.no_model_step:
+        p_ms, p_wall = preact18_stack_step(_hip, args.steps, args.warmup)
+        call('tt_empty_cache')
+        d_ms, d_wall = dcgan_generator_step(_hip, args.steps, args.warmup)
+        call('tt_empty_cache')
+        # convolution FLOPs of one pass (2*N*K*C*R*S*P*Q summed over the layers); forward, input
+        # gradient and weight gradient each count it once
+        stacks = {'preact_resnet18_stack': {
+                      'metric': 'PreAct-ResNet-18 basic-block stack fwd+bwd (conv + BatchNorm + ReLU + shortcuts)',
+                      'config': {'workload': 'batch 128, 3x32x32, 20 convolutions, 142.19 GFLOP per pass'},
+                      'ms_per_step': round(p_wall, 3), 'gpu_ms_per_step': round(p_ms, 3),
+                      'conv_tflops_equivalent': round(3 * 142.19e9 / (p_wall * 1e-3) / 1e12, 2)},
+                  'dcgan_generator_stack': {
+                      'metric': 'DCGAN generator fwd+bwd (ConvTranspose2d + BatchNorm + ReLU)',
+                      'config': {'workload': 'batch 128, latent 100 -> 3x64x64, 5 transposed convolutions, '
+                                             '26.78 GFLOP per pass'},
+                      'ms_per_step': round(d_wall, 3), 'gpu_ms_per_step': round(d_ms, 3),
+                      'conv_tflops_equivalent': round(3 * 26.78e9 / (d_wall * 1e-3) / 1e12, 2)},
+                  'note': 'whole stacks, every kernel counted in the time, only convolution FLOPs in the rate; '
+                          'the input of the first layer needs no gradient, so its input-gradient pass does not run'}
+
     # ---- what the device sustains on the two bounding resources, measured in this run ----------
     mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
     hbm_read, hbm_copy = _hip.probe_hbm(2 << 30)
@@ -504,6 +598,7 @@ def main():
                     'elementwise_gbs_at_same_size': act,
                     'cpu_baseline': cpu_pool},
         'resnet50_step': model,
+        'stacks': stacks,
     }
     print(json.dumps(out))
 
