@@ -350,6 +350,9 @@ def main():
     ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
     ap.add_argument('--model-step-only', action='store_true',
                     help='run only the whole-network ResNet-50 training step and print its object (for profiling)')
+    ap.add_argument('--stack-only', choices=('preact', 'dcgan'),
+                    help='run only the PreAct-ResNet-18 stack or the DCGAN generator stack and print its object '
+                         '(for profiling)')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this path runs on exactly one GPU (asked for --gpus {args.gpus}); '
@@ -366,6 +369,16 @@ def main():
     info = _hip.device_info()
     call = _hip.call
     rng = np.random.default_rng(0)
+    if args.stack_only:
+        fn = preact18_stack_step if args.stack_only == 'preact' else dcgan_generator_step
+        gflop = 142.19 if args.stack_only == 'preact' else 26.78
+        s_ms, s_wall = fn(_hip, args.steps, args.warmup)
+        print(json.dumps({'metric': f'{args.stack_only} stack fwd+bwd through the module API', 'value': round(s_wall, 3),
+                          'unit': 'ms', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                          'ms_per_step': round(s_wall, 3), 'gpu_ms_per_step': round(s_ms, 3),
+                          'higher_is_better': False, 'dtype': 'f32', 'data': 'synthetic',
+                          'conv_tflops_equivalent': round(3 * gflop * 1e9 / (s_wall * 1e-3) / 1e12, 2)}))
+        return
     if args.model_step_only:
         ips, m_ms, m_wall, m_losses = resnet50_train_step(_hip, args.steps, args.warmup)
         print(json.dumps({'metric': 'ResNet-50 training step images/s (module API)', 'value': round(ips, 1),
