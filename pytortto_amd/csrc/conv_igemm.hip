@@ -179,6 +179,7 @@ __global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ 
 // not have that tap).  Worth it only when Cg is tiny: the zero taps are wasted MACs.
 struct PackDense {
   int Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, HxWx, Wx;
+  int cellW;   // pixel classes per cell row (a multiple of sw)
 };
 __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restrict__ wp, PackDense a,
                                    KEntry* __restrict__ tab, KTabArgs ta, int4* __restrict__ rowtab) {
@@ -187,7 +188,7 @@ __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restr
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= a.Ipad) return;
   const int cls = i / a.Cg, c = i % a.Cg;
-  const int ch = cls / a.sw, cw = cls % a.sw;
+  const int ch = cls / a.cellW, cw = cls % a.cellW;
   if (kq == 0 && i < a.I) rowtab[i] = make_int4(c * a.HxWx + ch * a.Wx + cw, ch, cw, c);
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (i < a.I) {
@@ -1147,27 +1148,49 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
 
   if (groups == 1 && classes > 1 && classes * Cg <= 64 && Hx >= sh && Wx >= sw) {
     // tiny Cg: per-class GEMMs would fill 3 of 32 MFMA rows; stack all classes as rows instead
-    int amin = 1 << 30, amax = -(1 << 30), bmin = 1 << 30, bmax = -(1 << 30);
-    for (int ch = 0; ch < sh; ++ch)
-      for (int r = 0; r < R; ++r)
-        if (((ch + ph - r * dh) % sh + sh) % sh == 0) {
-          const int a = (ch + ph - r * dh) / sh;   // exact
-          amin = a < amin ? a : amin;
-          amax = a > amax ? a : amax;
+    // A cell of the output is one period of the stride pattern, or a few of them side by side:
+    // fh x fw periods make sh*fh x sw*fw pixel classes, each Cg rows of the GEMM.  More classes
+    // fill more of the 32 or 64 tile rows, at the price of a union tap window one dy pixel
+    // larger per added period; the cell with the fewest tile MACs per output pixel is taken.
+    auto window = [](int cell, int stride, int pad, int taps, int dil, int* lo, int* hi) {
+      *lo = 1 << 30;
+      *hi = -(1 << 30);
+      for (int cc = 0; cc < cell; ++cc)
+        for (int r = 0; r < taps; ++r)
+          if (((cc + pad - r * dil) % stride + stride) % stride == 0) {
+            const int a = (cc + pad - r * dil) / stride;   // exact
+            *lo = a < *lo ? a : *lo;
+            *hi = a > *hi ? a : *hi;
+          }
+    };
+    int fh = 1, fw = 1;
+    {
+      long long best = -1;
+      for (int th = 1; th <= 2; ++th)
+        for (int tw = 1; tw <= 4; tw *= 2) {
+          const int rows = sh * th * sw * tw * Cg;
+          if (rows > 64 || Hx < sh * th || Wx < sw * tw) continue;
+          int lo, hi, lo2, hi2;
+          window(sh * th, sh, ph, R, dh, &lo, &hi);
+          window(sw * tw, sw, pw, S, dw, &lo2, &hi2);
+          if (lo > hi || lo2 > hi2) continue;
+          const long long taps = (long long)(hi - lo + 1) * (hi2 - lo2 + 1);
+          if ((th > 1 || tw > 1) && taps > 31) continue;   // wider cells only while the tap-mask mode holds them
+          // tile MACs per output pixel, scaled by 8 so that the division by the cell size is exact
+          const long long cost = (rows <= 32 ? 32 : 64) * taps * (8 / (th * tw));
+          if (best < 0 || cost < best) { best = cost; fh = th; fw = tw; }
         }
-    for (int cw = 0; cw < sw; ++cw)
-      for (int s2 = 0; s2 < S; ++s2)
-        if (((cw + pw - s2 * dw) % sw + sw) % sw == 0) {
-          const int b = (cw + pw - s2 * dw) / sw;
-          bmin = b < bmin ? b : bmin;
-          bmax = b > bmax ? b : bmax;
-        }
+    }
+    const int cellH = sh * fh, cellW = sw * fw;
+    int amin, amax, bmin, bmax;
+    window(cellH, sh, ph, R, dh, &amin, &amax);
+    window(cellW, sw, pw, S, dw, &bmin, &bmax);
     if (amin <= amax && bmin <= bmax) {
       const int Na = amax - amin + 1, Nb = bmax - bmin + 1;
-      const int I = classes * Cg;
+      const int I = cellH * cellW * Cg;
       const int Kred = Kg * Na * Nb;
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
-      const int U = ceil_div(Hx, sh), V = ceil_div(Wx, sw);
+      const int U = ceil_div(Hx, cellH), V = ceil_div(Wx, cellW);
       const int M = N * U * V;
       TileChoice t;
       t.bm = I <= 32 ? 32 : 64;
@@ -1191,17 +1214,17 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       p.I = I; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
       p.divUV = tt::make_fastdiv((uint32_t)(U * V));
       p.divV = tt::make_fastdiv((uint32_t)V);
-      p.su = 1; p.bh = amin; p.sv = 1; p.bw = bmin;
+      p.su = fh; p.bh = amin; p.sv = fw; p.bw = bmin;
       p.Hlim = P; p.Wlim = Q; p.srcRow = Q;
       p.srcStrideN = K * P * Q; p.srcStrideG = 0;
       p.outStrideN = C * Hx * Wx; p.outStrideG = 0; p.outStrideI = 0; p.outRow = Wx;
-      p.ou = sh; p.ouh = 0; p.ov = sw; p.ovw = 0;
+      p.ou = cellH; p.ouh = 0; p.ov = cellW; p.ovw = 0;
       p.rowtab = rowtab; p.outH = Hx; p.outW = Wx;
       KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1, 0, 0};
       choose_mode(p, ka, false, N, U, V, (long long)wp_bytes);
       {
         tt::ProfScope prof(TT_PROF_CONV_PREP);
-        PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx};
+        PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx, cellW};
         pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa, tab, ka, rowtab);
         TT_LAUNCH_CHECK();
       }
