@@ -1137,6 +1137,13 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
   TT_REQUIRE_INIT();
   TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
   if (check_common("tt_conv2d_dgrad_f32", N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+  // One dy pixel per image spread over a whole R x S kernel (the first layer of a transposed
+  // generator: latent vector -> R x S map): every dx pixel has exactly one tap, tap (h, w), so
+  // dx[n][(c,h,w)] = sum_k dy[n][k] * w[k][(c,h,w)] is the input gradient of a 1x1 convolution
+  // with C*R*S channels on 1x1 images.  As R x S taps it would run R*S times the products.
+  if (P == 1 && Q == 1 && R * S > 1 && ph == 0 && pw == 0 && dh == 1 && dw == 1 && Hx == R && Wx == S && groups == 1 &&
+      bias == nullptr && tt::fits_i32((long long)C * R * S))
+    return conv2d_dgrad(dy, w, nullptr, dx, N, C * R * S, 1, 1, K, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1, 1, size_only);
   const int Cg = C / groups, Kg = K / groups;
   const int gh = gcd(sh, dh), gw = gcd(sw, dw);
   const int rstep = sh / gh, sstep = sw / gw;   // valid taps of a class: r0, r0+rstep, ...

@@ -122,6 +122,8 @@ CONVT_TILE_CASES = [
     (16, 100, 1, 1, 512, 4, 4, (1, 1), (0, 0), (0, 0), (1, 1), 1),   # DCGAN layer 1 (reduced batch)
     (8, 256, 8, 8, 128, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),    # DCGAN upsampling layer
     (8, 64, 16, 16, 3, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1),     # DCGAN last layer: 3 output channels
+    (130, 24, 1, 1, 40, 3, 5, (2, 3), (0, 0), (0, 0), (1, 1), 1),    # 1x1 input, rectangular kernel, stride irrelevant: one matrix product
+    (4, 24, 1, 1, 40, 3, 3, (2, 2), (0, 0), (1, 1), (1, 1), 1),      # 1x1 input with output padding: not that case
 ]
 
 
@@ -150,6 +152,10 @@ def test_conv_transpose_forward_backward(case):
     dw = ops.conv2d_wgrad(gyd, xd, w.shape, st, pd, dl, g)
     db = ops.channel_sum(gyd)
     _check('y', y.get(), y32, y64)
+    # without a bias (a 1x1 input spread over the whole kernel then runs as one matrix product)
+    y0 = ops.conv2d_dgrad(xd, wd, None, y32.shape[-2:], st, pd, dl, g)
+    bb, bb64 = b.reshape(1, -1, 1, 1), b.astype(np.float64).reshape(1, -1, 1, 1)
+    _check('y without bias', y0.get(), y32 - bb, y64 - bb64)
     _check('dx', dx.get(), dx32, dx64)
     _check('dw', dw.get(), dw32, dw64, reduction=True)
     _check('db', db.get(), db32, db64, reduction=True)
