@@ -28,6 +28,7 @@ PROTOTYPES = {
     'tt_sync': [],
     'tt_set_conv_math': [_I],
     'tt_get_conv_math': [POINTER(c_int)],
+    'tt_set_conv_dense_cell_min_tiles': [_I],
     'tt_event_create': [POINTER(c_void_p)],
     'tt_event_record': [_P],
     'tt_event_elapsed_ms': [_P, _P, POINTER(c_float)],

@@ -1060,9 +1060,18 @@ int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// tt_set_conv_dense_cell_min_tiles: tiles per CU a larger dense input-gradient cell must leave
+int g_dense_cell_min_tiles = 4;
+
 }  // namespace
 
 extern "C" {
+
+int tt_set_conv_dense_cell_min_tiles(int tiles_per_cu) {
+  TT_REQUIRE(tiles_per_cu >= 0 && tiles_per_cu <= 1024, "tt_set_conv_dense_cell_min_tiles: %d is out of range (0..1024)", tiles_per_cu);
+  g_dense_cell_min_tiles = tiles_per_cu;
+  return 0;
+}
 
 // `size_only`: report the workspace bytes this call would ask the library for and do nothing else.
 static int conv2d_fwd(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
@@ -1172,21 +1181,29 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
     };
     int fh = 1, fw = 1;
     {
+      // equal costs: the taller cell first (its stores keep the narrower column stride)
+      static const int kCells[6][2] = {{1, 1}, {2, 1}, {1, 2}, {2, 2}, {1, 4}, {2, 4}};
       long long best = -1;
-      for (int th = 1; th <= 2; ++th)
-        for (int tw = 1; tw <= 4; tw *= 2) {
-          const int rows = sh * th * sw * tw * Cg;
-          if (rows > 64 || Hx < sh * th || Wx < sw * tw) continue;
-          int lo, hi, lo2, hi2;
-          window(sh * th, sh, ph, R, dh, &lo, &hi);
-          window(sw * tw, sw, pw, S, dw, &lo2, &hi2);
-          if (lo > hi || lo2 > hi2) continue;
-          const long long taps = (long long)(hi - lo + 1) * (hi2 - lo2 + 1);
-          if ((th > 1 || tw > 1) && taps > 31) continue;   // wider cells only while the tap-mask mode holds them
-          // tile MACs per output pixel, scaled by 8 so that the division by the cell size is exact
-          const long long cost = (rows <= 32 ? 32 : 64) * taps * (8 / (th * tw));
-          if (best < 0 || cost < best) { best = cost; fh = th; fw = tw; }
+      for (const auto& cell : kCells) {
+        const int th = cell[0], tw = cell[1];
+        const int rows = sh * th * sw * tw * Cg;
+        if (rows > 64 || Hx < sh * th || Wx < sw * tw) continue;
+        int lo, hi, lo2, hi2;
+        window(sh * th, sh, ph, R, dh, &lo, &hi);
+        window(sw * tw, sw, pw, S, dw, &lo2, &hi2);
+        if (lo > hi || lo2 > hi2) continue;
+        const long long taps = (long long)(hi - lo + 1) * (hi2 - lo2 + 1);
+        if (th > 1 || tw > 1) {
+          if (taps > 31) continue;   // larger cells only while the tap-mask mode holds their window
+          // and only while four tiles per CU remain: with fewer, the blocks of a CU no longer
+          // cover each other's stalls and the saved MACs are lost again (measured)
+          const long long cells = (long long)N * ceil_div(Hx, sh * th) * ceil_div(Wx, sw * tw);
+          if (cells < 256LL * g_dense_cell_min_tiles * kCUs) continue;
         }
+        // tile MACs per output pixel, scaled by 8 so that the division by the cell size is exact
+        const long long cost = (rows <= 32 ? 32 : 64) * taps * (8 / (th * tw));
+        if (best < 0 || cost < best) { best = cost; fh = th; fw = tw; }
+      }
     }
     const int cellH = sh * fh, cellW = sw * fw;
     int amin, amax, bmin, bmax;

@@ -95,6 +95,18 @@ def test_conv_tile_configurations(case):
     _run_conv(case, seed=1)
 
 
+@pytest.mark.parametrize('case', [c for c in TILE_CASES if c[1] <= 5 and c[7] != (1, 1)])
+def test_conv_dense_input_gradient_with_every_cell_shape(case):
+    """Strided layers with very few input channels: without the tile-count threshold these small
+    inputs take the larger cells (several stride periods per cell) of the dense input gradient."""
+    from pytortto_amd import _hip
+    _hip.call('tt_set_conv_dense_cell_min_tiles', 0)
+    try:
+        _run_conv(case, seed=3)
+    finally:
+        _hip.call('tt_set_conv_dense_cell_min_tiles', 4)
+
+
 # Images too large for 32-bit byte offsets relative to a tile's (a chunk's) first image: the
 # kernels must fall back from buffer addressing to 64-bit addresses with compared bounds.
 LARGE_IMAGE_CASES = [
