@@ -94,6 +94,10 @@ struct Igemm {
   // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
   const int4* rowtab;
   int outH, outW;
+  // strided 1x1 input gradients: only one pixel of every sh x 2 cell of dx has a tap.  > 0: the
+  // launch stores each value together with the zero to its right (one 8-byte store) and zero
+  // pairs into the cellFill - 1 rows below, so dx needs no clearing beforehand
+  int cellFill;
   // stream-K launches only: the tiles*chunks reduction steps are dealt evenly to the blocks
   int skDpTiles;             // tiles [0, skDpTiles) are computed whole, block b takes b, b+blocks, ...
   int skBlocks;              // blocks that share the remaining tiles' reduction steps
@@ -214,6 +218,7 @@ __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restr
 // tiles, row tiles fastest, so blocks that share a pixel tile (same gathered operand) share an L2.
 using tt::xcd_remap;
 
+typedef float floatx2 __attribute__((ext_vector_type(2)));
 constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2;
 constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format
 constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out of range and read 0
@@ -593,6 +598,31 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
       // (1x1 layers) spend a noticeable share of their time here otherwise.
       const int i0u = __builtin_amdgcn_readfirstlane(i0);
       const uint32_t hoff = (uint32_t)(4 * h * p.outStrideI);
+      if (p.cellFill > 0) {
+#pragma unroll
+        for (int y = 0; y < NT; ++y) {
+          if (mok[y]) {
+            const uint32_t vo = obase[y] + hoff;
+#pragma unroll
+            for (int x = 0; x < MT; ++x) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int srow = i0u + (wm * MT + x) * 32 + 8 * q;
+                if (srow < p.I) {
+#pragma unroll
+                  for (int j = 0; j < 4; ++j) {
+                    float* __restrict__ rowp = p.out + (size_t)(srow + j) * (size_t)p.outStrideI;
+                    *reinterpret_cast<floatx2*>(rowp + vo) = floatx2{acc[x][y][4 * q + j], 0.f};
+                    for (int f = 1; f < p.cellFill; ++f)
+                      *reinterpret_cast<floatx2*>(rowp + vo + (uint32_t)(f * p.outRow)) = floatx2{0.f, 0.f};
+                  }
+                }
+              }
+            }
+          }
+        }
+        return;
+      }
 #pragma unroll
       for (int y = 0; y < NT; ++y) {
         if (mok[y]) {
@@ -825,7 +855,15 @@ __global__ __launch_bounds__(kThreads) void igemm_fixup(const Igemm p) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int i = i0 + (wm * MT + x) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-    if (i < p.I) p.out[obase + (uint32_t)(i * p.outStrideI)] = acc[r >> 2][r & 3] + bz[r];
+    if (i < p.I) {
+      float* __restrict__ o = p.out + obase + (uint32_t)(i * p.outStrideI);
+      if (p.cellFill > 0) {   // no bias in these launches
+        *reinterpret_cast<floatx2*>(o) = floatx2{acc[r >> 2][r & 3], 0.f};
+        for (int f = 1; f < p.cellFill; ++f) *reinterpret_cast<floatx2*>(o + f * p.outRow) = floatx2{0.f, 0.f};
+      } else {
+        *o = acc[r >> 2][r & 3] + bz[r];
+      }
+    }
   }
 }
 
@@ -1273,7 +1311,13 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
   // Parity classes without a tap hold only bias (or zero).  Without a bias it is cheaper to
   // clear dx once with a streaming fill than to launch a strided store kernel per empty class.
   bool prefilled = false;
-  if (bias == nullptr) {
+  // 1x1 kernels with a stride two wide: the one class that has a tap stores whole cells instead
+  const int cell_fill = (bias == nullptr && R == 1 && S == 1 && ph == 0 && pw == 0 && sw == 2 && sh <= 4 &&
+                         Hx == P * sh && Wx == Q * sw && Cg % 8 == 0 && (reinterpret_cast<uintptr_t>(dx) & 7) == 0)
+                            ? sh : 0;
+  if (cell_fill > 0) {
+    prefilled = true;   // the classes without a tap have nothing left to do
+  } else if (bias == nullptr) {
     bool any_empty = false;
     for (int ch = 0; ch < sh && ch < Hx; ++ch) {
       bool has = false;
@@ -1343,6 +1387,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       p.outStrideN = C * Hx * Wx; p.outStrideG = Cg * Hx * Wx; p.outStrideI = Hx * Wx; p.outRow = Wx;
       p.ou = sh; p.ouh = ch; p.ov = sw; p.ovw = cw;
       p.kStride = P * Q;   // 1x1 layers: dx[c][n,hw] = sum_k w[k][c] * dy[n][k][hw]
+      p.cellFill = cell_fill;
       p.Kred = Kred;
       if (KQ > 0) {
         // h = u*sh + ch reads dy row (h + ph - r0*dh)/sh = u + (ch + ph - r0*dh)/sh  (exact)

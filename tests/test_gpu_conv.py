@@ -80,7 +80,10 @@ TILE_CASES = [
     (3, 16, 14, 14, 16, 6, 6, (1, 1), (2, 2), (1, 1), 1),       # 36 taps > 31: compare-and-select addressing in all three passes
     (2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1),       # padded 1x1: not the plain-GEMM geometry, one-tap mask
     (4, 48, 10, 10, 24, 3, 3, (1, 1), (0, 0), (1, 1), 1),       # unpadded 3x3, rows (24) and weight rows shorter than a tile
-    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)    # tiny C with stride > 1: the input gradient stacks the pixel classes of a cell of one or more stride periods as GEMM rows
+    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)    (8, 64, 18, 20, 32, 1, 1, (3, 2), (0, 0), (1, 1), 1),        # strided 1x1, whole cells: the input gradient stores value + zeros of a 3x2 cell itself
+    (4, 40, 15, 14, 24, 1, 1, (2, 2), (0, 0), (1, 1), 1),        # strided 1x1, last row of dx not covered by the forward: cleared beforehand instead
+    (4, 32, 12, 12, 16, 1, 1, (2, 2), (0, 0), (1, 1), 2),        # strided 1x1 with groups
+    # tiny C with stride > 1: the input gradient stacks the pixel classes of a cell of one or more stride periods as GEMM rows
     (3, 3, 45, 43, 16, 7, 7, (2, 2), (3, 3), (1, 1), 1),        # stem taps, odd image: cells two periods wide, ragged last cell and last column
     (2, 1, 21, 30, 8, 3, 3, (2, 2), (1, 1), (1, 1), 1),         # one channel: cells widened both ways
     (2, 2, 17, 19, 8, 4, 4, (2, 2), (1, 1), (1, 1), 1),         # 4x4 stride 2 (the transposed generator's taps), rows left uncovered by the forward
