@@ -372,7 +372,7 @@ def main():
     if args.stack_only:
         fn = preact18_stack_step if args.stack_only == 'preact' else dcgan_generator_step
         gflop = 142.19 if args.stack_only == 'preact' else 26.78
-        s_ms, s_wall = fn(_hip, args.steps, args.warmup)
+        s_ms, s_wall = fn(_hip, args.steps, args.warmup)   # the full run uses at least 50 steps after 20 warm-up steps
         print(json.dumps({'metric': f'{args.stack_only} stack fwd+bwd through the module API', 'value': round(s_wall, 3),
                           'unit': 'ms', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
                           'ms_per_step': round(s_wall, 3), 'gpu_ms_per_step': round(s_ms, 3),
@@ -519,9 +519,12 @@ def main():
     # ---- the other two stack configurations, through the module API -----------------------------
     stacks = None
     if not args.no_model_step:
-        p_ms, p_wall = preact18_stack_step(_hip, args.steps, args.warmup)
+        # steps of 1-6 ms: enough of them that the first ones (pool refill after tt_empty_cache, clock
+        # ramp after the host-side pause) do not set the figure
+        s_steps, s_warmup = max(args.steps, 50), max(args.warmup, 20)
+        p_ms, p_wall = preact18_stack_step(_hip, s_steps, s_warmup)
         call('tt_empty_cache')
-        d_ms, d_wall = dcgan_generator_step(_hip, args.steps, args.warmup)
+        d_ms, d_wall = dcgan_generator_step(_hip, s_steps, s_warmup)
         call('tt_empty_cache')
         # convolution FLOPs of one pass (2*N*K*C*R*S*P*Q summed over the layers); forward, input
         # gradient and weight gradient each count it once
