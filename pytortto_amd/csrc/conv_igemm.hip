@@ -911,11 +911,6 @@ TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k
   t.bm = I <= 64 ? 64 : 128;
   t.bn = I <= 64 ? 256 : 128;
   if (small && groups == 1) { t.bm = 64; t.bn = 64; }
-  if (const char* e = getenv("TT_IGEMM_TILE")) {   // tuning knob: 0 = 128x128, 1 = 64x256
-    if (e[0] == '0') { t.bm = 128; t.bn = 128; }
-    if (e[0] == '1') { t.bm = 64; t.bn = 256; }
-    if (e[0] == '2') { t.bm = 64; t.bn = 64; }
-  }
   t.sk_blocks = 0;
   const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
   if (allow_stream_k && wants_stream_k(tiles, chunks, groups)) {
