@@ -101,10 +101,10 @@ int tt_get_conv_math(int* mode);   /* host pointer */
  * Such launches stack the pixel classes of a cell of the output (one period of the stride
  * pattern, or two / four periods side by side) as rows of one matrix product; a larger cell
  * wastes fewer multiplications but leaves fewer tiles.  A larger cell is taken only while at
- * least `tiles_per_cu` tiles per compute unit remain (default 4; 0 = always, which lets small
- * inputs reach every cell shape).  Results do not depend on it beyond summation order.
- * Process-wide, applies to later calls. */
-int tt_set_conv_dense_cell_min_tiles(int tiles_per_cu);
+ * least `tiles` tiles of 256 cells remain (default 384 = 1.5 per compute unit; 0 = always, which
+ * lets small inputs reach every cell shape).  Results do not depend on it beyond summation
+ * order.  Process-wide, applies to later calls. */
+int tt_set_conv_dense_cell_min_tiles(int tiles);
 
 /* y[N,K,P,Q] = conv(x[N,C,H,W], w[K,C/groups,R,S]) (+ bias[K] if not NULL).
  * Replaces _padding + _sliding_window_view + einsum and the bias add:

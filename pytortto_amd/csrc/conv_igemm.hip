@@ -1093,16 +1093,16 @@ int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// tt_set_conv_dense_cell_min_tiles: tiles per CU a larger dense input-gradient cell must leave
-int g_dense_cell_min_tiles = 4;
+// tt_set_conv_dense_cell_min_tiles: 256-pixel tiles a larger dense input-gradient cell must leave
+int g_dense_cell_min_tiles = 3 * kCUs / 2;
 
 }  // namespace
 
 extern "C" {
 
-int tt_set_conv_dense_cell_min_tiles(int tiles_per_cu) {
-  TT_REQUIRE(tiles_per_cu >= 0 && tiles_per_cu <= 1024, "tt_set_conv_dense_cell_min_tiles: %d is out of range (0..1024)", tiles_per_cu);
-  g_dense_cell_min_tiles = tiles_per_cu;
+int tt_set_conv_dense_cell_min_tiles(int tiles) {
+  TT_REQUIRE(tiles >= 0 && tiles <= (1 << 20), "tt_set_conv_dense_cell_min_tiles: %d is out of range (0..2^20)", tiles);
+  g_dense_cell_min_tiles = tiles;
   return 0;
 }
 
@@ -1228,10 +1228,10 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
         const long long taps = (long long)(hi - lo + 1) * (hi2 - lo2 + 1);
         if (th > 1 || tw > 1) {
           if (taps > 31) continue;   // larger cells only while the tap-mask mode holds their window
-          // and only while four tiles per CU remain: with fewer, the blocks of a CU no longer
-          // cover each other's stalls and the saved MACs are lost again (measured)
+          // and only while about 1.5 tiles per CU remain: with fewer, too few blocks are resident to
+          // cover each other's load latency and the saved MACs are lost again (measured)
           const long long cells = (long long)N * ceil_div(Hx, sh * th) * ceil_div(Wx, sw * tw);
-          if (cells < 256LL * g_dense_cell_min_tiles * kCUs) continue;
+          if (cells < 256LL * g_dense_cell_min_tiles) continue;
         }
         // tile MACs per output pixel, scaled by 8 so that the division by the cell size is exact
         const long long cost = (rows <= 32 ? 32 : 64) * taps * (8 / (th * tw));

@@ -107,7 +107,7 @@ def test_conv_dense_input_gradient_with_every_cell_shape(case):
     try:
         _run_conv(case, seed=3)
     finally:
-        _hip.call('tt_set_conv_dense_cell_min_tiles', 4)
+        _hip.call('tt_set_conv_dense_cell_min_tiles', 384)
 
 
 # Images too large for 32-bit byte offsets relative to a tile's (a chunk's) first image: the
