@@ -102,7 +102,7 @@ int tt_get_conv_math(int* mode);   /* host pointer */
  * pattern, or two / four periods side by side) as rows of one matrix product; a larger cell
  * wastes fewer multiplications but leaves fewer tiles.  A larger cell is taken only while at
  * least `tiles` tiles of 256 cells remain (default 384 = 1.5 per compute unit; 0 = always, which
- * lets small inputs reach every cell shape).  Results do not depend on it beyond summation
+ * lets small inputs reach the larger cells).  Results do not depend on it beyond summation
  * order.  Process-wide, applies to later calls. */
 int tt_set_conv_dense_cell_min_tiles(int tiles);
 

@@ -90,6 +90,8 @@ TILE_CASES = [
     (2, 3, 20, 22, 8, 5, 3, (3, 2), (2, 1), (1, 1), 1),         # stride 3 x 2: 18 classes x 3 channels stay in one period
     (2, 2, 19, 21, 8, 3, 3, (2, 2), (2, 2), (2, 2), 1),         # dilation shares a factor with the stride: classes without taps
     (2, 5, 16, 9, 8, 3, 5, (2, 2), (1, 2), (1, 1), 1),          # five channels, image narrower than a four-period cell
+    (4, 3, 3, 40, 8, 3, 3, (2, 2), (1, 1), (1, 1), 1),          # image too low for a taller cell: two periods wide instead
+    (4, 1, 3, 40, 8, 3, 3, (2, 2), (1, 1), (1, 1), 1),          # the same with one channel: four periods wide
 ]
 
 
@@ -99,9 +101,10 @@ def test_conv_tile_configurations(case):
 
 
 @pytest.mark.parametrize('case', [c for c in TILE_CASES if c[1] <= 5 and c[7] != (1, 1)])
-def test_conv_dense_input_gradient_with_every_cell_shape(case):
+def test_conv_dense_input_gradient_with_larger_cells(case):
     """Strided layers with very few input channels: without the tile-count threshold these small
-    inputs take the larger cells (several stride periods per cell) of the dense input gradient."""
+    inputs take the larger cells (several stride periods per cell) of the dense input gradient;
+    between them the cases take cells of 2x1, 1x2, 2x2, 1x4 and 2x4 periods."""
     from pytortto_amd import _hip
     _hip.call('tt_set_conv_dense_cell_min_tiles', 0)
     try:
