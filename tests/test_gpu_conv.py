@@ -80,7 +80,11 @@ TILE_CASES = [
     (3, 16, 14, 14, 16, 6, 6, (1, 1), (2, 2), (1, 1), 1),       # 36 taps > 31: compare-and-select addressing in all three passes
     (2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1),       # padded 1x1: not the plain-GEMM geometry, one-tap mask
     (4, 48, 10, 10, 24, 3, 3, (1, 1), (0, 0), (1, 1), 1),       # unpadded 3x3, rows (24) and weight rows shorter than a tile
-    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)    (8, 64, 18, 20, 32, 1, 1, (3, 2), (0, 0), (1, 1), 1),        # strided 1x1, whole cells: the input gradient stores value + zeros of a 3x2 cell itself
+    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)
+    (8, 64, 18, 20, 32, 1, 1, (3, 2), (0, 0), (1, 1), 1),       # strided 1x1, whole cells: the input gradient stores value + zeros of a 3x2 cell itself
+    (4, 64, 16, 12, 64, 1, 1, (4, 2), (0, 0), (1, 1), 1),       # the same with cells four rows high (the tallest the whole-cell stores take)
+    (8, 256, 28, 28, 512, 1, 1, (2, 2), (0, 0), (1, 1), 1),     # whole cells with the reduction of every tile split between blocks: the second stage stores the cells
+    (48, 128, 21, 28, 256, 1, 1, (3, 2), (0, 0), (1, 1), 1),    # split reduction and cells three rows high
     (4, 40, 15, 14, 24, 1, 1, (2, 2), (0, 0), (1, 1), 1),        # strided 1x1, last row of dx not covered by the forward: cleared beforehand instead
     (4, 32, 12, 12, 16, 1, 1, (2, 2), (0, 0), (1, 1), 2),        # strided 1x1 with groups
     # tiny C with stride > 1: the input gradient stacks the pixel classes of a cell of one or more stride periods as GEMM rows
@@ -93,6 +97,14 @@ TILE_CASES = [
     (4, 3, 3, 40, 8, 3, 3, (2, 2), (1, 1), (1, 1), 1),          # image too low for a taller cell: two periods wide instead
     (4, 1, 3, 40, 8, 3, 3, (2, 2), (1, 1), (1, 1), 1),          # the same with one channel: four periods wide
 ]
+
+
+def test_tile_case_list_is_complete():
+    """A case that slips into the comment of the line above it would silently drop out."""
+    assert len(TILE_CASES) == 36
+    assert all(len(c) == 11 for c in TILE_CASES)
+    strided_1x1 = [c for c in TILE_CASES if c[5:7] == (1, 1) and c[7] != (1, 1) and c[10] == 1]
+    assert {c[7][0] for c in strided_1x1} == {2, 3, 4}      # cells two, three and four rows high
 
 
 @pytest.mark.parametrize('case', TILE_CASES)
