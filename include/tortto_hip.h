@@ -153,6 +153,22 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
                         float* running_mean_out, float* running_var_out,
                         double momentum, double eps, int N, int C, int HW);
 
+/* tt_bn_fwd_train_f32 for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments, same kernels and bit-identical results, but the first sweep's per-channel partial
+ * moments go to a fixed 256 KiB array in the library's device image instead of the workspace that
+ * grows on demand, launches are never bracketed for tt_profile_read, and the call makes no
+ * hipMalloc / hipFree / event creation.  Limit: tt_workspace_size_bn_f32(...) <= 262144 bytes
+ * (16384 partial moments; every tensor of at most 2^29 elements fits); beyond that the call fails
+ * with a message and launches nothing.  All calls on one device share the array: it needs no
+ * clearing between calls (every slot read was written by the same call), but calls that overlap on
+ * one device race.  tt_init() looks the array's device address up once per device. */
+int tt_bn_fwd_train_noalloc_f32(const float* x, const float* gamma, const float* beta, float* y,
+                                float* save_mean, float* save_var_eps, float* save_sd,
+                                const float* running_mean_in, const float* running_var_in,
+                                float* running_mean_out, float* running_var_out,
+                                double momentum, double eps, int N, int C, int HW);
+
 /* Normalisation with given statistics (eval mode), autograd/grad_nn.py:931-959:
  * save_* are written from mean[C]/var[C] exactly as in training so that backward can follow. */
 int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, float* y,

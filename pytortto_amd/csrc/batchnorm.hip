@@ -675,22 +675,55 @@ __global__ __launch_bounds__(tt::kWave) void channel_sum_finish(const double2* _
   if (threadIdx.x == 0) out[blockIdx.x] = (float)a;
 }
 
+// ---- fixed scratch for the entry point that allocates nothing -----------------------------------
+// tt_bn_fwd_train_noalloc_f32 keeps the first sweep's partial moments here instead of in the
+// library workspace: one double2 per (channel, reduction split), 256 KiB per device for the life
+// of the process (enough for every tensor of at most 2^29 elements).  The array's name is only a host-side handle; its device address is looked up once
+// per device (tt::bn_scratch_init, called by tt_init with that device current) and everything on
+// the host uses that address.  Every slot a launch reads was written by the reduce kernel of the
+// same call, so nothing needs clearing between calls; calls that overlap on one device would race.
+constexpr int kScratchPartials = 16384;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) double2 scratch[kScratchPartials];
+double2* g_scratch_ptr[kMaxDevices] = {};
+
 }  // namespace
+
+namespace tt {
+
+int bn_scratch_init(int device) {
+  TT_REQUIRE(device >= 0 && device < kMaxDevices, "device index %d beyond the %d the scratch table covers", device,
+             kMaxDevices);
+  if (g_scratch_ptr[device]) return 0;
+  double2* ptr = nullptr;
+  TT_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+  TT_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the BatchNorm scratch array");
+  g_scratch_ptr[device] = ptr;
+  return 0;
+}
+
+}  // namespace tt
 
 extern "C" {
 
-int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
-                        float* save_var_eps, float* save_sd, const float* running_mean_in,
+// Training forward behind both entry points.  `fixed_partials` == nullptr: the partial moments of
+// the first sweep go to the library workspace (grown on demand) and launches are bracketed for
+// tt_profile_read.  Otherwise they go to that buffer of `fixed_capacity` entries and the call makes
+// no allocation of any kind (no workspace growth, no event creation).
+static int bn_fwd_train(const char* fn, const float* x, const float* gamma, const float* beta, float* y,
+                        float* save_mean, float* save_var_eps, float* save_sd, const float* running_mean_in,
                         const float* running_var_in, float* running_mean_out, float* running_var_out,
-                        double momentum, double eps, int N, int C, int HW) {
+                        double momentum, double eps, int N, int C, int HW, double2* fixed_partials,
+                        size_t fixed_capacity) {
   TT_REQUIRE_INIT();
-  if (check_shape("tt_bn_fwd_train_f32", N, C, HW)) return -1;
-  TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "tt_bn_fwd_train_f32: null tensor pointer");
+  if (check_shape(fn, N, C, HW)) return -1;
+  TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
   const long long m = (long long)N * HW;
   TT_REQUIRE(m > 1, "Expected more than 1 value per channel when training, got input size [%d, %d, %d]", N, C, HW);
   const bool track = running_mean_in && running_var_in;
-  TT_REQUIRE(!track || (running_mean_out && running_var_out),
-             "tt_bn_fwd_train_f32: running statistics given without output buffers");
+  TT_REQUIRE(!track || (running_mean_out && running_var_out), "%s: running statistics given without output buffers",
+             fn);
+  const bool timed = fixed_partials == nullptr;
   FwdArgs a{};
   a.x = x; a.gamma = gamma; a.beta = beta; a.y = y;
   a.save_mean = save_mean; a.save_var_eps = save_var_eps; a.save_sd = save_sd;
@@ -703,7 +736,7 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   a.eps = (float)eps;
   hipStream_t st = tt::stream();
   if (const int cap = small_channel_capacity(N, C, HW)) {
-    tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
+    tt::ProfScope prof(timed ? TT_PROF_BN_FWD_APPLY : -1);
     const Geometry gs = small_geometry(N, C, HW);
     if (cap == 16) bn_fwd_small<16><<<C, kThreads, 0, st>>>(a, gs);
     else bn_fwd_small<kSmallMax><<<C, kThreads, 0, st>>>(a, gs);
@@ -714,24 +747,56 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   int mode, rmode;
   plan(N, C, HW, &g, &mode);
   plan_reduce(N, C, HW, &gr, &rmode);
-  void* ws;
-  if (tt::workspace(sizeof(double2) * (size_t)C * gr.splits, &ws)) return -1;
+  const size_t partials = (size_t)C * gr.splits;
+  double2* part = fixed_partials;
+  if (part) {
+    TT_REQUIRE(partials <= fixed_capacity,
+               "%s: [%d, %d, %d] needs %zu partial moments, the fixed scratch array holds %zu "
+               "(use tt_bn_fwd_train_f32, whose workspace grows)",
+               fn, N, C, HW, partials, fixed_capacity);
+  } else {
+    void* ws;
+    if (tt::workspace(sizeof(double2) * partials, &ws)) return -1;
+    part = (double2*)ws;
+  }
   dim3 grid(g.splits, C);
   {
-    tt::ProfScope prof(TT_PROF_BN_FWD_REDUCE);
-    launch_reduce<0>(rmode, dim3(gr.splits, C), x, x, nullptr, (double2*)ws, gr);
+    tt::ProfScope prof(timed ? TT_PROF_BN_FWD_REDUCE : -1);
+    launch_reduce<0>(rmode, dim3(gr.splits, C), x, x, nullptr, part, gr);
   }
   TT_LAUNCH_CHECK();
-  a.partial = (const double2*)ws;
+  a.partial = part;
   a.partial_splits = gr.splits;
   {
-    tt::ProfScope prof(TT_PROF_BN_FWD_APPLY);
+    tt::ProfScope prof(timed ? TT_PROF_BN_FWD_APPLY : -1);
     if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
     if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
     if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
   }
   TT_LAUNCH_CHECK();
   return 0;
+}
+
+int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
+                        float* save_var_eps, float* save_sd, const float* running_mean_in,
+                        const float* running_var_in, float* running_mean_out, float* running_var_out,
+                        double momentum, double eps, int N, int C, int HW) {
+  return bn_fwd_train("tt_bn_fwd_train_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd, running_mean_in,
+                      running_var_in, running_mean_out, running_var_out, momentum, eps, N, C, HW, nullptr, 0);
+}
+
+int tt_bn_fwd_train_noalloc_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
+                                float* save_var_eps, float* save_sd, const float* running_mean_in,
+                                const float* running_var_in, float* running_mean_out, float* running_var_out,
+                                double momentum, double eps, int N, int C, int HW) {
+  TT_REQUIRE_INIT();
+  int dev = -1;
+  TT_HIP(hipGetDevice(&dev));
+  TT_REQUIRE(dev >= 0 && dev < kMaxDevices && g_scratch_ptr[dev] != nullptr,
+             "tt_bn_fwd_train_noalloc_f32: the scratch array of device %d was not set up by tt_init", dev);
+  return bn_fwd_train("tt_bn_fwd_train_noalloc_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd,
+                      running_mean_in, running_var_in, running_mean_out, running_var_out, momentum, eps, N, C, HW,
+                      g_scratch_ptr[dev], (size_t)kScratchPartials);
 }
 
 int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, float* y, const float* mean,

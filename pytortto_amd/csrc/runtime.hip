@@ -105,7 +105,7 @@ int workspace(size_t bytes, void** out) {
 
 ProfScope::ProfScope(int kernel_id) : id(kernel_id), start(nullptr) {
   State& s = S();
-  if (!s.profiling) return;
+  if (!s.profiling || kernel_id < 0) return;   // a negative id: this launch is never timed
   hipEvent_t e = nullptr;
   if (!s.event_pool.empty()) {
     e = s.event_pool.back();
@@ -166,6 +166,7 @@ int tt_init(int device) {
   TT_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
              "libtortto_hip is built for gfx950 (MI355X) only; device %d is %s", device, prop.gcnArchName);
   TT_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
+  if (tt::bn_scratch_init(device)) return -1;   // device address of the fixed scratch array, once per device
   s.device = device;
   s.ready = true;
   return 0;

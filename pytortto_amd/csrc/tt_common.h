@@ -21,7 +21,12 @@ bool initialised();
 // more; work on the stream is ordered, so consecutive launches may reuse it.
 int workspace(size_t bytes, void** out);
 
-// Brackets the launches made during its lifetime with events when profiling is enabled.
+// Looks up the device address of the fixed scratch array behind tt_bn_fwd_train_noalloc_f32 for
+// `device`, which must be the current device (batchnorm.hip).  Called once per device by tt_init.
+int bn_scratch_init(int device);
+
+// Brackets the launches made during its lifetime with events when profiling is enabled
+// (a negative kernel id switches it off for that scope).
 struct ProfScope {
   explicit ProfScope(int kernel_id);
   ~ProfScope();
