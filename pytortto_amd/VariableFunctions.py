@@ -58,23 +58,16 @@ def mean(input, dim=None, keepdim=False):
 
 
 def flatten(x, start_dim=0, end_dim=-1):
-    """VariableFunctions.py:108-127."""
-    shape = x.shape
-    if end_dim < 0:
-        end_dim = len(shape) + end_dim
-    end_dim += 1
-    if start_dim < 0:
-        start_dim = len(shape) + start_dim
-    if start_dim >= end_dim:
+    """Collapse dimensions ``start_dim`` .. ``end_dim`` (inclusive, negative values count from the
+    end) into one (interface of VariableFunctions.py:108-127).  Returns ``x`` itself when nothing
+    would change, else a view."""
+    rank = len(x.shape)
+    first, last = start_dim % rank if rank else 0, end_dim % rank if rank else 0
+    if first > last:
         raise RuntimeError('flatten() has invalid args: start_dim cannot come after end_dim')
-    newshape = shape[:start_dim]
-    if start_dim != end_dim:
-        newshape += (-1,)
-    if end_dim < len(shape):
-        newshape += shape[end_dim:]
-    if len(newshape) != len(shape):
-        return x.view(newshape)
-    return x
+    if first == last:
+        return x
+    return x.view(x.shape[:first] + (-1,) + x.shape[last + 1:])
 
 
 def mm(input, mat2):

@@ -85,9 +85,19 @@ class Add(Function):
         g, = grad_outputs
         sa, sb = ctx.params['shapes']
         if g.__class__ is hiparray:
-            def back(shape):
-                return g if shape == g.shape else ops.sum_rows(g, prod(shape)).reshape(shape)
-            return (back(sa) if ctx.needs_input_grad[0] else None), (back(sb) if ctx.needs_input_grad[1] else None)
+            # Every operand receives an array of its own, as the reference's reverse_broadcast does
+            # (its ``sum((), keepdims=True)`` copies): gradients are stored by reference further on
+            # and some backward functions scale theirs in place (LeakyRelu, grad_nn.py:92-94), so a
+            # shared array would hand one branch the other's already-masked gradient.
+            need_a, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+
+            def back(shape, fresh):
+                if shape != g.shape:
+                    return ops.sum_rows(g, prod(shape)).reshape(shape)
+                return g.copy() if fresh else g
+            ga = back(sa, False) if need_a else None
+            gb = back(sb, need_a and sa == g.shape) if need_b else None
+            return ga, gb
         return (_unbroadcast(g, sa) if ctx.needs_input_grad[0] else None,
                 _unbroadcast(g, sb) if ctx.needs_input_grad[1] else None)
 

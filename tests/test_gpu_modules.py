@@ -317,3 +317,49 @@ def test_workspace_queries_bound_what_the_calls_request():
     assert workspace_now() == 0
     with pytest.raises(RuntimeError, match='not divisible by groups'):
         query('tt_workspace_size_conv2d_fwd_f32', n, c, h, h, k, r, r, st, st, pd, pd, 1, 1, 7)
+
+
+def _device_leaf(values):
+    import pytortto_amd as tt
+    from pytortto_amd.xparray import hiparray
+    return tt.Tensor(hiparray(np.ascontiguousarray(values, dtype=np.float32)), requires_grad=True)
+
+
+def test_add_backward_gives_each_operand_its_own_gradient_array():
+    """``Add`` hands every operand a gradient array of its own, as the reference's
+    ``reverse_broadcast`` does (helper.py:32-42: ``sum((), keepdims=True)`` copies).  LeakyReLU's
+    backward scales the array it is given in place (grad_nn.py:92-94), so with a shared array one
+    branch would receive the other's already-scaled gradient."""
+    import pytortto_amd as tt
+    from pytortto_amd.nn import functional as F
+    rng = np.random.default_rng(5)
+    a, b = rng.standard_normal((3, 4, 5, 6)), rng.standard_normal((3, 4, 5, 6))
+    g = rng.standard_normal((3, 4, 5, 6)).astype(np.float32)
+    slope = 0.25
+
+    at, bt = _device_leaf(a), _device_leaf(b)
+    out = F.leaky_relu(at, slope) + F.leaky_relu(bt, slope)
+    out.backward(tt.tensor(g).cuda())
+    ga_ref = g * np.where(a.astype(np.float32) >= 0, np.float32(1), np.float32(slope))
+    gb_ref = g * np.where(b.astype(np.float32) >= 0, np.float32(1), np.float32(slope))
+    assert np.array_equal(at.grad.get(), ga_ref)
+    assert np.array_equal(bt.grad.get(), gb_ref)
+
+    # a residual add whose skip operand is consumed after the LeakyReLU branch scaled its gradient
+    xt = _device_leaf(a)
+    h = F.leaky_relu(xt, slope)
+    out = F.leaky_relu(h, 0.5) + h
+    out.backward(tt.tensor(g).cuda())
+    h_ref = np.maximum(a.astype(np.float32) * np.float32(slope), a.astype(np.float32))
+    gh = g * np.where(h_ref >= 0, np.float32(1), np.float32(0.5)) + g
+    gx_ref = gh * np.where(a.astype(np.float32) >= 0, np.float32(1), np.float32(slope))
+    np.testing.assert_allclose(xt.grad.get(), gx_ref, rtol=1e-6, atol=0)
+
+    # two leaves of one shape: their .grad are distinct buffers, so accumulating into one
+    # (a second backward pass) leaves the other alone
+    at, bt = _device_leaf(a), _device_leaf(b)
+    (at + bt).backward(tt.tensor(g).cuda())
+    assert at.grad.ptr != bt.grad.ptr
+    (at + at).backward(tt.tensor(g).cuda())
+    assert np.array_equal(bt.grad.get(), g)
+    assert np.array_equal(at.grad.get(), g + (g + g))
