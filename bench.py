@@ -100,11 +100,64 @@ class BnLayer:
         self.dg, self.db = hiparray.empty((c,)), hiparray.empty((c,))
         self.dims = (n, c, h * w)
 
-    def run(self, call):
+    def run_fwd(self, call):
         call('tt_bn_fwd_train_f32', self.x.ptr, self.gamma.ptr, self.beta.ptr, self.y.ptr, self.mean.ptr,
              self.var.ptr, self.sd.ptr, self.rm.ptr, self.rv.ptr, self.rm.ptr, self.rv.ptr, 0.1, 1e-5, *self.dims)
+
+    def run_bwd(self, call):
         call('tt_bn_bwd_f32', self.x.ptr, self.dy.ptr, self.gamma.ptr, self.mean.ptr, self.var.ptr, self.sd.ptr,
              self.dx.ptr, self.dg.ptr, self.db.ptr, *self.dims)
+
+    def run(self, call):
+        self.run_fwd(call)
+        self.run_bwd(call)
+
+
+def bn_passes_separately(hip, call, bns, steps, cold):
+    """Forward and backward of every BatchNorm shape bracketed by their own HIP events.  With
+    `cold`, 2.3 GB are streamed through the device between the passes (an elementwise add over
+    three 768 MB arrays, outside the events), so a pass finds none of its tensors in the 256 MB
+    memory-side cache -- the way a network, which runs other layers in between, meets it.  Without,
+    the passes follow each other directly on the same tensors, as in the headline figure."""
+    from pytortto_amd.xparray import hiparray
+    fa = fb = None
+    if cold:
+        n = 192 << 20
+        fa, fb = hiparray.empty((n,)), hiparray.empty((n,))
+        call('tt_fill_f32', fa.ptr, 1.0, n)
+        call('tt_fill_f32', fb.ptr, 0.0, n)
+
+    def flush():
+        if cold:
+            call('tt_add_f32', fa.ptr, fb.ptr, fb.ptr, fa.size)
+
+    out = {}
+    for b in bns:
+        pairs = []
+        for it in range(steps + 2):
+            flush()
+            e0 = hip.Event().record()
+            b.run_fwd(call)
+            e1 = hip.Event().record()
+            flush()
+            e2 = hip.Event().record()
+            b.run_bwd(call)
+            e3 = hip.Event().record()
+            if it >= 2:
+                pairs.append((e0, e1, e2, e3))
+        hip.synchronize()
+        fwd = sum(e0.elapsed_ms(e1) for e0, e1, _, _ in pairs) / steps
+        bwd = sum(e2.elapsed_ms(e3) for _, _, e2, e3 in pairs) / steps
+        out['x'.join(map(str, b.shape))] = {
+            'fwd_ms': round(fwd, 4), 'bwd_ms': round(bwd, 4),
+            'fwd_gbs': round(3 * b.bytes / (fwd * 1e-3) / 1e9, 1), 'bwd_gbs': round(5 * b.bytes / (bwd * 1e-3) / 1e9, 1),
+            'fwd_bwd_gbs': round(8 * b.bytes / ((fwd + bwd) * 1e-3) / 1e9, 1)}
+    total_bytes = sum(8 * b.bytes for b in bns)
+    total_ms = sum(v['fwd_ms'] + v['bwd_ms'] for v in out.values())
+    out['both_shapes_fwd_bwd_gbs'] = round(total_bytes / (total_ms * 1e-3) / 1e9, 1)
+    out['both_shapes_pct_of_peak'] = round(100 * total_bytes / (total_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 1)
+    del fa, fb
+    return out
 
 
 def timed_steps(hip, step, steps, warmup):
@@ -130,6 +183,34 @@ def profiled_steps(hip, step, steps):
     prof = hip.profile_read()
     hip.profile_enable(False)
     return prof
+
+
+def per_layer_table(hip, call, layers, reps):
+    """Forward, input gradient and weight gradient of every unique ResNet-50 shape timed on their own
+    (HIP events on the library stream around `reps` back-to-back calls after 3 warm-up calls; the
+    weight gradient includes its float64 reduce, the input gradient its weight repack).  The
+    per-layer roofline is min(fp32 MFMA peak, AI * 8 TB/s) with AI = F / (4 * (|x| + |w| + |y|)):
+    the three passes of a layer move the same three tensors' worth of bytes."""
+    rows = []
+    for l in layers:
+        c, h, k, r, s, p, count = l.spec
+        a = l.args
+        passes = {
+            'fwd': lambda: call('tt_conv2d_fwd_f32', l.x.ptr, l.w.ptr, None, l.y.ptr, *a),
+            'dgrad': lambda: call('tt_conv2d_dgrad_f32', l.dy.ptr, l.w.ptr, None, l.dx.ptr, *a, l.q, l.q),
+            'wgrad': lambda: call('tt_conv2d_wgrad_f32', l.x.ptr, l.dy.ptr, l.dw.ptr, *a, l.q, l.q),
+        }
+        nbytes = 4.0 * (l.x.size + l.w.size + l.y.size)
+        ai = l.flops / nbytes
+        roof = min(PEAK_FP32_MFMA_TFLOPS, ai * PEAK_HBM_GBS / 1e3)
+        row = {'shape': f'{c}x{h}x{h}->{k} k{r} s{s} p{p}', 'count': count, 'gflop': round(l.flops / 1e9, 2),
+               'ai_flop_per_byte': round(ai, 1), 'roofline_tflops': round(roof, 1)}
+        for name, fn in passes.items():
+            ms, _ = timed_steps(hip, fn, reps, 3)
+            tf = l.flops / (ms * 1e-3) / 1e12
+            row[name] = {'ms': round(ms, 4), 'tflops': round(tf, 1), 'frac_of_roofline': round(tf / roof, 3)}
+        rows.append(row)
+    return rows
 
 
 def resnet50_train_step(hip, steps, warmup, batch=BATCH):
@@ -321,6 +402,24 @@ def cpu_baseline_conv(batch):
     return flops, seconds
 
 
+def cpu_baseline_c1(reps=5):
+    """Oracle forward + backward of the single-layer baseline configuration at its full size:
+    Conv2d(16, 32, 3, padding=1, bias) on x [32,16,32,32].  (flops counted, median seconds)"""
+    import oracle
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((32, 16, 32, 32), dtype=np.float32)
+    w = rng.uniform(-1 / 12, 1 / 12, (32, 16, 3, 3)).astype(np.float32)
+    b = rng.uniform(-1 / 12, 1 / 12, 32).astype(np.float32)
+    dy = rng.standard_normal((32, 32, 32, 32), dtype=np.float32)
+    times = []
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        _, xpad = oracle.convolution_forward(x, w, b, (1, 1), (1, 1), (1, 1), 1)
+        oracle.convolution_backward(dy, x, xpad, w, (1, 1), (1, 1), (1, 1), 1)
+        times.append(time.perf_counter() - t0)
+    return 3 * 2.0 * 32 * 32 * 16 * 9 * 32 * 32, float(np.median(times[1:]))
+
+
 def cpu_baseline_bn(batch_div):
     import oracle
     rng = np.random.default_rng(0)
@@ -350,6 +449,8 @@ def main():
     ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
     ap.add_argument('--model-step-only', action='store_true',
                     help='run only the whole-network ResNet-50 training step and print its object (for profiling)')
+    ap.add_argument('--per-layer-only', action='store_true',
+                    help='print only the per-layer table of the 23 ResNet-50 convolution shapes (for profiling)')
     ap.add_argument('--stack-only', choices=('preact', 'dcgan'),
                     help='run only the PreAct-ResNet-18 stack or the DCGAN generator stack and print its object '
                          '(for profiling)')
@@ -392,6 +493,12 @@ def main():
     layers = [ConvLayer(spec, BATCH, rng) for spec in RESNET50_CONVS]
     flops_per_pass = sum(l.flops * l.count for l in layers)
     assert abs(flops_per_pass / 1e9 - 523.15) < 0.05, flops_per_pass
+    if args.per_layer_only:
+        rows = per_layer_table(_hip, call, layers, max(args.steps, 20))
+        print(json.dumps({'metric': 'per-layer conv fwd / dgrad / wgrad of the 23 unique ResNet-50 shapes, batch 64',
+                          'unit': 'ms, TFLOP/s', 'n_gpus': 1, 'steps': max(args.steps, 20), 'warmup': 3,
+                          'dtype': 'f32', 'data': 'synthetic', 'per_layer': rows}))
+        return
 
     def conv_step():
         for l in layers:
@@ -410,6 +517,7 @@ def main():
     n_wg, ms_wg = prof['conv_wgrad']
     wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
     kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
+    layer_rows = per_layer_table(_hip, call, layers, 20)
 
     # optional reduced-precision variant, reported separately and never part of `value`: the three
     # passes on bf16 MFMA (operands rounded inside the kernels, fp32 accumulation and tensors)
@@ -458,6 +566,8 @@ def main():
     # dominant kernel: bn_bwd_apply (reads x, dy, writes dx: 3*S algorithmic bytes per launch)
     n_ba, ms_ba = bprof['bn_bwd_apply']
     bwd_apply_gbs = sum(3 * b.bytes for b in bns) * args.steps / (ms_ba * 1e-3) / 1e9
+    bn_warm = bn_passes_separately(_hip, call, bns, args.steps, cold=False)
+    bn_cold = bn_passes_separately(_hip, call, bns, args.steps, cold=True)
     del bns
     call('tt_empty_cache')
 
@@ -555,9 +665,14 @@ def main():
         cpu_conv = {'value': round(f / sec / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
                     'sample': f'oracle fwd+dgrad+wgrad once over the 23 unique ResNet-50 conv shapes at batch '
                               f'{cbatch} ({f / 1e9:.0f} GFLOP counted, {sec:.1f} s)'}
-        nb, sec = cpu_baseline_bn(2)
+        f1, sec1 = cpu_baseline_c1()
+        cpu_conv['single_layer_config_full_size'] = {
+            'value': round(f1 / sec1 / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
+            'sample': f'oracle Conv2d(16,32,3,padding=1) fwd+bwd on x [32,16,32,32], the CPU-runnable configuration at '
+                      f'full size ({f1 / 1e9:.2f} GFLOP counted, median of 5 runs {sec1 * 1e3:.1f} ms)'}
+        nb, sec = cpu_baseline_bn(1)
         cpu_bn = {'value': round(nb / sec / 1e9, 3), 'unit': 'GB/s', 'cores': cores, 'kind': 'port',
-                  'sample': f'oracle BatchNorm fwd+bwd at both shapes with batch/2 ({nb / 1e9:.2f} GB counted, '
+                  'sample': f'oracle BatchNorm fwd+bwd at both shapes, full batch ({nb / 1e9:.2f} GB counted, '
                             f'{sec:.1f} s)'}
 
     out = {
@@ -582,6 +697,9 @@ def main():
                      'avg_launch_ms': round((ms_fwd + ms_dg) / max(1, n_fwd + n_dg), 5)},
         'kernels_ms_per_step': kernel_ms,
         'wgrad_tflops': round(wgrad_tflops, 2),
+        'per_layer': {'what': 'each unique shape and pass timed alone, 20 back-to-back calls after 3 warm-up calls; '
+                              'roofline_tflops = min(157.3, AI * 8 TB/s), AI = F / (4 * (|x| + |w| + |y|))',
+                      'rows': layer_rows},
         'conv_bf16_variant': bf16_variant,
         'cpu_baseline': cpu_conv,
         'bn': {'metric': 'BatchNorm2d training fwd+bwd GB/s', 'value': round(bn_gbs, 1), 'unit': 'GB/s',
@@ -590,6 +708,10 @@ def main():
                'config': {'workload': 'BatchNorm2d train fwd+bwd fp32 NCHW at [64,256,56,56] and [128,64,112,112], '
                                       'x ~ N(2,3), 8*S algorithmic bytes per shape'},
                'per_shape_gbs': per_shape,
+               'passes_back_to_back': bn_warm,
+               'passes_cold_cache': dict(bn_cold, what='2.3 GB streamed through the device before each pass, outside '
+                                                       'the events: no tensor of the pass is left in the 256 MB '
+                                                       'memory-side cache; `value` above is the back-to-back figure'),
                'roofline': {'bound': 'hbm', 'kernel': 'bn_bwd_apply (reads x, dy; writes dx)',
                             'achieved': round(bwd_apply_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                             'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4),

@@ -11,6 +11,10 @@
  *     message.  Nothing throws or aborts across this boundary.
  *   - all tensor pointers are DEVICE pointers to C-contiguous float32 NCHW data unless a
  *     parameter is documented as a host pointer.  Outputs are caller-allocated.
+ *   - tensor pointers of the convolution, BatchNorm, pooling and elementwise entry points must be
+ *     16-byte aligned (the kernels use 16-byte vector accesses; tt_malloc blocks are 256-byte
+ *     aligned); a misaligned pointer is refused with an error.  Exception: x and dy of
+ *     tt_conv2d_wgrad_f32 may have any 4-byte alignment (it falls back to scalar fetches).
  *   - kernels are enqueued on one library-owned HIP stream and return immediately;
  *     tt_sync() / tt_memcpy_d2h() wait for them.  One caller thread at a time.
  *   - tensors are limited to 2^31-1 elements each (32-bit element offsets in the kernels);

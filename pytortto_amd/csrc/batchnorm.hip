@@ -718,6 +718,7 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
   TT_REQUIRE_INIT();
   if (check_shape(fn, N, C, HW)) return -1;
   TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
+  TT_REQUIRE_ALIGNED(fn, x, y);
   const long long m = (long long)N * HW;
   TT_REQUIRE(m > 1, "Expected more than 1 value per channel when training, got input size [%d, %d, %d]", N, C, HW);
   const bool track = running_mean_in && running_var_in;
@@ -806,6 +807,7 @@ int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, fl
   if (check_shape("tt_bn_fwd_eval_f32", N, C, HW)) return -1;
   TT_REQUIRE(x && y && mean && var && save_mean && save_var_eps && save_sd,
              "tt_bn_fwd_eval_f32: null tensor pointer");
+  TT_REQUIRE_ALIGNED("tt_bn_fwd_eval_f32", x, y);
   Geometry g;
   int mode;
   plan(N, C, HW, &g, &mode);
@@ -832,6 +834,7 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const flo
   TT_REQUIRE_INIT();
   if (check_shape("tt_bn_bwd_f32", N, C, HW)) return -1;
   TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "tt_bn_bwd_f32: null tensor pointer");
+  TT_REQUIRE_ALIGNED("tt_bn_bwd_f32", x, dy, dx);
   if (!dx && !dgamma && !dbeta) return 0;
   if (const int cap = small_channel_capacity(N, C, HW)) {
     tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
@@ -870,6 +873,7 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
   TT_REQUIRE_INIT();
   if (check_shape("tt_channel_sum_f32", N, K, HW)) return -1;
   TT_REQUIRE(t && out, "tt_channel_sum_f32: null tensor pointer");
+  TT_REQUIRE_ALIGNED("tt_channel_sum_f32", t);
   Geometry g;
   int mode;
   plan_reduce(N, K, HW, &g, &mode);

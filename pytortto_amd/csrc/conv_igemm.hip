@@ -877,18 +877,20 @@ struct TileChoice {
   int sk_blocks;   // > 0: persistent launch with this many blocks, left-over tiles split stream-K fashion
 };
 
-constexpr int kCUs = 256;             // MI355X
-constexpr int kSkBlocks = 2 * kCUs;   // persistent launches: two blocks per CU (three or four measured slower)
+// Compute units of the device (256 on an MI355X), and the blocks of a persistent launch: two per
+// CU (three or four measured slower).
+int cus() { return tt::compute_units(); }
+int sk_blocks_f32() { return 2 * cus(); }
 
 // Stream-K pays (a second small kernel, partial tiles through HBM) and only helps when the
 // tiles do not spread evenly over the CUs; it needs a reduction long enough to split.
 bool wants_stream_k(long long tiles, int chunks, int groups) {
   if (groups != 1 || chunks < 8) return false;
   // many tiles and a short reduction: hardware block scheduling balances better than fixed rounds
-  if (tiles >= 3LL * kSkBlocks && chunks < 64) return false;
-  if (tiles * chunks < 4LL * kSkBlocks) return false;
-  const long long rounds = (tiles + kCUs - 1) / kCUs;
-  return (double)tiles / (double)(rounds * kCUs) < 0.93;
+  if (tiles >= 3LL * sk_blocks_f32() && chunks < 64) return false;
+  if (tiles * chunks < 4LL * sk_blocks_f32()) return false;
+  const long long rounds = (tiles + cus() - 1) / cus();
+  return (double)tiles / (double)(rounds * cus()) < 0.93;
 }
 
 // The bf16 kernels are bound by their fetch path, not by the matrix pipe: smaller tiles fetch more
@@ -897,8 +899,7 @@ bool bf16_math() { return tt::conv_math() == TT_CONV_MATH_BF16; }
 
 // Blocks of a persistent launch: the bf16 kernels hide their loads with a third block per CU
 // (measured: 3 % faster than two, four do not fit the register file).
-constexpr int kSkBlocksBf16 = 3 * kCUs;
-int sk_launch_blocks() { return bf16_math() ? kSkBlocksBf16 : kSkBlocks; }
+int sk_launch_blocks() { return bf16_math() ? 3 * cus() : sk_blocks_f32(); }
 
 // 128x128 by default, 64 rows when a group has no more than 64 of them.  When that leaves
 // CUs idle or unevenly loaded the reduction is split stream-K fashion; if it is too short for
@@ -915,7 +916,7 @@ TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k
   const long long tiles = (long long)ceil_div(I, t.bm) * ceil_div(M, t.bn);
   if (allow_stream_k && wants_stream_k(tiles, chunks, groups)) {
     t.sk_blocks = sk_launch_blocks();
-  } else if (tiles * groups < kCUs) {
+  } else if (tiles * groups < cus()) {
     t.bm = 64;
     t.bn = 64;
     const long long small = (long long)ceil_div(I, 64) * ceil_div(M, 64);
@@ -1094,7 +1095,9 @@ int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // tt_set_conv_dense_cell_min_tiles: 256-pixel tiles a larger dense input-gradient cell must leave
-int g_dense_cell_min_tiles = 3 * kCUs / 2;
+// (< 0: not set, 1.5 per compute unit)
+int g_dense_cell_min_tiles = -1;
+int dense_cell_min_tiles() { return g_dense_cell_min_tiles >= 0 ? g_dense_cell_min_tiles : 3 * cus() / 2; }
 
 }  // namespace
 
@@ -1111,6 +1114,7 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
                       int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, size_t* size_only) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
+  TT_REQUIRE_ALIGNED("tt_conv2d_fwd_f32", x, w, y);
   const int P = (H + 2 * ph - dh * (R - 1) - 1) / sh + 1;
   const int Q = (W + 2 * pw - dw * (S - 1) - 1) / sw + 1;
   TT_REQUIRE(H + 2 * ph - dh * (R - 1) - 1 >= 0 && W + 2 * pw - dw * (S - 1) - 1 >= 0,
@@ -1178,6 +1182,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
                         int Q, size_t* size_only) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
+  TT_REQUIRE_ALIGNED("tt_conv2d_dgrad_f32", dy, w, dx);
   if (check_common("tt_conv2d_dgrad_f32", N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
   // One dy pixel per image spread over a whole R x S kernel (the first layer of a transposed
   // generator: latent vector -> R x S map): every dx pixel has exactly one tap, tap (h, w), so
@@ -1231,7 +1236,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
           // and only while about 1.5 tiles per CU remain: with fewer, too few blocks are resident to
           // cover each other's load latency and the saved MACs are lost again (measured)
           const long long cells = (long long)N * ceil_div(Hx, sh * th) * ceil_div(Wx, sw * tw);
-          if (cells < 256LL * g_dense_cell_min_tiles) continue;
+          if (cells < 256LL * dense_cell_min_tiles()) continue;
         }
         // tile MACs per output pixel, scaled by 8 so that the division by the cell size is exact
         const long long cost = (rows <= 32 ? 32 : 64) * taps * (8 / (th * tw));

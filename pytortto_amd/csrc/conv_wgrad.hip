@@ -532,6 +532,7 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
   TT_REQUIRE_INIT();
   const char* fn = "tt_conv2d_wgrad_f32";
   TT_REQUIRE(x && dy && dw, "%s: null tensor pointer", fn);
+  TT_REQUIRE_ALIGNED(fn, dw);
   TT_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0 && P > 0 && Q > 0, "%s: sizes must be positive", fn);
   TT_REQUIRE(sh > 0 && sw > 0 && dh > 0 && dw_ > 0 && ph >= 0 && pw >= 0, "%s: stride/dilation must be positive, padding non-negative", fn);
   TT_REQUIRE(groups > 0 && groups <= 65535 && C % groups == 0 && K % groups == 0, "%s: channels (%d, %d) not divisible by groups=%d", fn, C, K, groups);
@@ -555,10 +556,10 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
   const int tilesI = ceil_div(Kg, bm), tilesJ = ceil_div(J, bn);
   const long long tiles = (long long)tilesI * tilesJ * groups;
   const int chunks = ceil_div(M, kBK);
-  // Two blocks fit a CU (LDS), so 512 run at a time and all take equally long: fill one round of
-  // 512 as well as possible, or two rounds if that fills them clearly better; at least 8 chunks
-  // (256 pixels) of work per split.
-  const int kSlots = 512;
+  // Two blocks fit a CU (LDS), so 2 x CUs (512 on an MI355X) run at a time and all take equally
+  // long: fill one such round as well as possible, or two rounds if that fills them clearly better;
+  // at least 8 chunks (256 pixels) of work per split.
+  const int kSlots = 2 * tt::compute_units();
   int splits = (int)(kSlots / tiles);
   const int two = (int)(2 * kSlots / tiles);
   if ((double)tiles * two / (2.0 * kSlots) > (double)tiles * splits / kSlots + 0.08) splits = two;

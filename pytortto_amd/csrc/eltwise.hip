@@ -17,7 +17,9 @@ __device__ __forceinline__ float apply1(float a, float b, float alpha) {
     return (t > a || t != t) ? t : a;
   }
   if (OP == kLeakyReluBwd) return b < 0.f ? a * alpha : a;   // a = dy, b = x: g[x < 0] *= slope, grad_nn.py:94
-  if (OP == kReluBwd) return b > 0.f ? a : 0.f;  // a = dy, b = y
+  // a = dy, b = y: the reference multiplies by the mask, gd0 * (yd0 > 0) (grad_nn.py:67), so a
+  // non-finite gradient at a masked element gives NaN and a negative one -0, not +0
+  if (OP == kReluBwd) return a * (b > 0.f ? 1.f : 0.f);
   if (OP == kAdd) return a + b;
   if (OP == kAxpy) return fmaf(alpha, a, b);      // a = v, b = acc
   if (OP == kAddScalar) return a + alpha;
@@ -70,9 +72,11 @@ int run(const char* fn, const float* a, const float* b, float* out, float alpha,
   TT_REQUIRE_INIT();
   if (n == 0) return 0;
   TT_REQUIRE(out != nullptr, "%s: null output pointer", fn);
+  TT_REQUIRE_ALIGNED(fn, a, b, out);
   size_t blocks = ((n >> 2) + kThreads - 1) / kThreads;
+  const size_t cap = (size_t)tt::compute_units() * 16;   // grid-stride beyond 16 blocks per CU
   if (blocks < 1) blocks = 1;
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks > cap) blocks = cap;
   eltwise<OP><<<(unsigned)blocks, kThreads, 0, tt::stream()>>>(a, b, out, alpha, n);
   TT_LAUNCH_CHECK();
   return 0;

@@ -180,7 +180,8 @@ __global__ __launch_bounds__(kThreads) void nll_loss_bwd(const float* __restrict
 unsigned blocks_for(size_t total) {
   size_t b = (total + kThreads - 1) / kThreads;
   if (b < 1) b = 1;
-  return (unsigned)(b < 256 * 16 ? b : 256 * 16);
+  const size_t cap = (size_t)tt::compute_units() * 16;
+  return (unsigned)(b < cap ? b : cap);
 }
 
 int check_rows(const char* fn, int R, int C) {

@@ -149,7 +149,8 @@ __global__ __launch_bounds__(kThreads) void adam_step_multi(AdamTensors ts, Adam
 
 unsigned blocks_for(size_t n) {
   size_t b = (n + kThreads - 1) / kThreads;
-  return (unsigned)(b < 256 * 16 ? b : 256 * 16);
+  const size_t cap = (size_t)tt::compute_units() * 16;
+  return (unsigned)(b < cap ? b : cap);
 }
 
 }  // namespace

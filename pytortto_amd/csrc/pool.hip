@@ -266,7 +266,7 @@ Band make_band(const Pool& g, int rows_fit, int cap) {
 
 unsigned grid_for(uint32_t total) {
   uint32_t blocks = (total + kThreads - 1) / kThreads;
-  const uint32_t cap = 256 * 32;
+  const uint32_t cap = (uint32_t)tt::compute_units() * 32;
   return blocks < cap ? blocks : cap;
 }
 
@@ -278,6 +278,7 @@ int tt_maxpool2d_fwd_f32(const float* x, float* y, int* tap, int NC, int H, int 
                          int sh, int sw, int ph, int pw, int dh, int dw) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(x && y && tap, "tt_maxpool2d_fwd_f32: null pointer");
+  TT_REQUIRE_ALIGNED("tt_maxpool2d_fwd_f32", x, y, tap);
   Pool g;
   if (int rc = fill("tt_maxpool2d_fwd_f32", &g, NC, H, W, P, Q, kh, kw, sh, sw, ph, pw, dh, dw)) return rc;
   const uint32_t total = (uint32_t)NC * P * Q;
@@ -302,6 +303,7 @@ int tt_maxpool2d_bwd_f32(const float* dy, const int* tap, float* dx, int NC, int
                          int kw, int sh, int sw, int ph, int pw, int dh, int dw) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(dy && tap && dx, "tt_maxpool2d_bwd_f32: null pointer");
+  TT_REQUIRE_ALIGNED("tt_maxpool2d_bwd_f32", dy, tap, dx);
   Pool g;
   if (int rc = fill("tt_maxpool2d_bwd_f32", &g, NC, H, W, P, Q, kh, kw, sh, sw, ph, pw, dh, dw)) return rc;
   const uint32_t total = (uint32_t)NC * H * W;

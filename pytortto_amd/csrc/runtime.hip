@@ -16,6 +16,7 @@ thread_local char g_err[512] = "";
 struct State {
   bool ready = false;
   int device = -1;
+  int compute_units = 256;
   hipStream_t stream = nullptr;
   // pooling allocator: freed blocks are kept per rounded size and handed out again, so the
   // autograd loop does not pay hipMalloc/hipFree (which synchronises the device) per tensor
@@ -79,6 +80,7 @@ int fail_hip(hipError_t e, const char* what, const char* file, int line) {
 }
 
 hipStream_t stream() { return S().stream; }
+int compute_units() { return S().compute_units; }
 int conv_math() { return S().conv_math; }
 bool initialised() { return S().ready; }
 
@@ -168,6 +170,7 @@ int tt_init(int device) {
   TT_HIP(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking));
   if (tt::bn_scratch_init(device)) return -1;   // device address of the fixed scratch array, once per device
   s.device = device;
+  s.compute_units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   s.ready = true;
   return 0;
 }

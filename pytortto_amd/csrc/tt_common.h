@@ -15,6 +15,9 @@ int fail_hip(hipError_t e, const char* what, const char* file, int line);
 // The one stream every kernel of the library is enqueued on.
 hipStream_t stream();
 bool initialised();
+// Compute units of the device tt_init() selected (256 on an MI355X): persistent grids, tile-count
+// thresholds and the caps on grid-stride launches scale with it.
+int compute_units();
 
 // Grow-only scratch memory owned by the library (split-K partial sums, repacked weights,
 // per-channel partial moments).  The pointer stays valid until the next call that asks for
@@ -74,6 +77,16 @@ __device__ __forceinline__ int xcd_remap(int b, int nb) {
   do {                                            \
     if (!(cond)) return tt::fail(-1, __VA_ARGS__); \
   } while (0)
+
+// Tensor pointers at the C ABI are 16-byte aligned (the kernels use 16-byte vector accesses);
+// null pointers (optional arguments) pass.
+namespace tt {
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+template <typename... P>
+inline bool all_aligned16(P... ptrs) { return (aligned16(ptrs) && ...); }
+}  // namespace tt
+#define TT_REQUIRE_ALIGNED(fn, ...) \
+  TT_REQUIRE(tt::all_aligned16(__VA_ARGS__), "%s: tensor pointers must be 16-byte aligned", fn)
 
 #define TT_REQUIRE_INIT() TT_REQUIRE(tt::initialised(), "tt_init() has not been called")
 

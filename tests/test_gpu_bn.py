@@ -6,15 +6,28 @@ import oracle
 
 pytestmark = pytest.mark.gpu
 
-# outputs and running statistics: rtol 1e-5 (plus an absolute floor for values that cancel to ~0:
-# two correct float32 evaluations of (x-mean)/sd*gamma+beta differ by ~1 ulp of the larger term)
+# outputs and running statistics: rtol 1e-5.  Two correct float32 evaluations of
+# (x-mean)/sd*gamma+beta differ by ~1 ulp of the larger term, so where the two terms cancel to a y
+# near zero the element-wise relative error has no bound; such elements -- and only such -- fall
+# back on an absolute floor of 2e-6 of the tensor's magnitude.  _close() checks that the floor is
+# used nowhere else: every element outside the pure rtol must be smaller than 5 % of the tensor's
+# magnitude, and in tensors of 4096 elements or more they must be fewer than 2 % of it (measured:
+# 0.1 - 1.0 % of y, where gamma * xhat and beta cancel to within a few percent; 2 - 4e-6 of dx).
 RTOL = 1e-5
 
 
 def _close(got, ref, rtol=RTOL, atol_scale=2e-6, name=''):
-    ref = np.asarray(ref)
+    """Returns the share of elements that needed the absolute floor."""
+    got, ref = np.asarray(got), np.asarray(ref)
     scale = float(np.abs(ref).max()) or 1.0
     np.testing.assert_allclose(got, ref, rtol=rtol, atol=atol_scale * scale, err_msg=name)
+    outside = np.abs(got - ref) > rtol * np.abs(ref)
+    share = float(outside.mean()) if outside.size else 0.0
+    if outside.any():
+        assert float(np.abs(ref[outside]).max()) <= 0.05 * scale, f'{name}: the floor was needed away from zero'
+        if ref.size >= 4096:
+            assert share <= 2e-2, f'{name}: {share:.2%} of the elements needed the floor'
+    return share
 
 
 def _inputs(shape, seed=0):
@@ -36,6 +49,8 @@ SHAPES = [
     (5, 7, 24, 20),      # plane kernel, ragged plane count per block
     (64, 64, 28, 28),    # plane kernel with several splits per channel
     (128, 4, 32, 32),    # few channels: maximum number of splits
+    # the BatchNorm shapes of the PreAct-ResNet-18 stack at its own batch size
+    (128, 64, 32, 32), (128, 128, 16, 16), (128, 256, 8, 8), (128, 512, 4, 4),
 ]
 
 
@@ -179,7 +194,7 @@ def test_bn_benchmark_shapes_full_size(shape):
     np.testing.assert_allclose(rv.get(), 0.9 + 0.1 * var64 * (m / (m - 1)), rtol=1e-5)
 
     y_ref, saved, rm_ref, rv_ref = oracle.batch_norm_forward(x, gamma, beta, rm0, rv0, True, 0.1, 1e-5)
-    _close(y, y_ref, name='y')
+    share_y = _close(y, y_ref, name='y')
     _close(rm.get(), rm_ref, name='running_mean')
     _close(rv.get(), rv_ref, name='running_var')
     np.testing.assert_allclose(y.mean(axis, dtype=np.float64), beta, atol=2e-6)
@@ -192,7 +207,9 @@ def test_bn_benchmark_shapes_full_size(shape):
     dg64 = (dy * xhat).sum(axis)
     np.testing.assert_allclose(db.get(), db64, rtol=1e-5, atol=1e-5 * np.abs(db64).max())
     np.testing.assert_allclose(dg.get(), dg64, rtol=1e-5, atol=1e-5 * np.abs(dg64).max())
-    _close(dx, dx_ref, rtol=1e-4, atol_scale=1e-5, name='dx')
+    share_dx = _close(dx, dx_ref, rtol=1e-4, atol_scale=1e-5, name='dx')
+    print(f'BatchNorm {shape}: share of elements outside the pure relative tolerance: y {share_y:.2e} (rtol 1e-5), '
+          f'dx {share_dx:.2e} (rtol 1e-4)')
     scale = float(np.abs(dx).sum(axis, dtype=np.float64).max())
     assert np.abs(dx.sum(axis, dtype=np.float64)).max() <= 1e-5 * scale
     assert np.abs((dx * xhat).sum(axis)).max() <= 1e-4 * scale          # exact only up to O(eps / var)
