@@ -138,6 +138,23 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw,
                         int sh, int sw, int ph, int pw, int dh, int dw_, int groups,
                         int P, int Q);
 
+/* Host-only checks of the index tables behind tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 (no
+ * counterpart in the reference; no device is needed and tt_init() need not have been called).
+ * The kernels turn a reduction index (c, r, s) -- (k, tap row, tap column) for the input gradient
+ * -- into an address through small per-geometry tables, which the library builds on the host,
+ * checks once per new geometry and keeps in device buffers of their own.  These calls run exactly
+ * that planning and check for a geometry without launching anything: every table entry, replayed
+ * for the extreme pixels under the kernel's own bounds rule, must address the element of x (dy)
+ * that autograd/grad_nn.py:603-611 (:659-682) pairs with that reduction index, inside the tensor.
+ * tt_conv2d_check_tables_selftest damages single entries and returns 0 when the check refuses each
+ * damaged table. */
+int tt_conv2d_check_tables_fwd_f32(int N, int C, int H, int W, int K, int R, int S,
+                                   int sh, int sw, int ph, int pw, int dh, int dw, int groups);
+int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R, int S,
+                                     int sh, int sw, int ph, int pw, int dh, int dw, int groups,
+                                     int P, int Q);
+int tt_conv2d_check_tables_selftest(void);
+
 /* out[K] = sum over n and the HW plane of t[N,K,HW]: the bias gradient gd0.sum((0,2,3)),
  * autograd/grad_nn.py:728, :774. */
 int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW);
@@ -192,8 +209,8 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
 /* Bytes of library workspace (repacked weights, index tables, partial sums) the corresponding call
  * asks for with the same geometry arguments; the library grows its workspace to the largest
  * request seen.  Same argument checks as the calls; nothing is launched or allocated.  The small
- * per-geometry tables the library caches separately (index tables, 16 bytes per output pixel for
- * the weight gradient) are not included. */
+ * per-geometry tables the library keeps in buffers of their own (index tables of a few KB, 16 bytes
+ * per output pixel for the weight gradient; released by tt_empty_cache) are not included. */
 int tt_workspace_size_conv2d_fwd_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S,
                                      int sh, int sw, int ph, int pw, int dh, int dw, int groups);
 int tt_workspace_size_conv2d_dgrad_f32(size_t* bytes, int N, int C, int Hx, int Wx, int K, int R, int S,

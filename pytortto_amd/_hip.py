@@ -40,6 +40,9 @@ PROTOTYPES = {
     'tt_conv2d_fwd_f32': [_P, _P, _P, _P] + [_I] * 14,
     'tt_conv2d_dgrad_f32': [_P, _P, _P, _P] + [_I] * 16,
     'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
+    'tt_conv2d_check_tables_fwd_f32': [_I] * 14,
+    'tt_conv2d_check_tables_dgrad_f32': [_I] * 16,
+    'tt_conv2d_check_tables_selftest': [],
     'tt_channel_sum_f32': [_P, _P, _I, _I, _I],
     'tt_workspace_size_conv2d_fwd_f32': [POINTER(c_size_t)] + [_I] * 14,
     'tt_workspace_size_conv2d_dgrad_f32': [POINTER(c_size_t)] + [_I] * 16,

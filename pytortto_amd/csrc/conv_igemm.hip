@@ -31,7 +31,9 @@
 // the operands rounded to bfloat16 after the LDS read and contracted by v_mfma_f32_32x32x16_bf16,
 // float32 accumulation, float32 tensors in memory.
 #include <cstdlib>
+#include <cstring>
 #include <map>
+#include <vector>
 
 #include "tt_common.h"
 
@@ -108,12 +110,15 @@ struct Igemm {
 // ---- preparation kernels (tiny) --------------------------------------------------------------
 
 // k -> {offset, steps}.  k = (a*TB + b)*TC + c:  off = a*sa + b*sb + c*sc, steps (b*stepH, c*stepW).
+// Tables are built on the host (host_ktab), checked there against the tensor they index
+// (check_ktab) and kept in device buffers of their own, one per geometry: no kernel writes them
+// and they never share memory with per-call scratch data.
 struct KTabArgs {
   int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
   int tapMask;   // 1: entries are {4*(off + offBias), tap number b*TC + c}
   int offBias;
 };
-__device__ __forceinline__ void write_ktab_entry(KEntry* __restrict__ tab, const KTabArgs& a, int k) {
+KEntry ktab_entry(const KTabArgs& a, int k) {
   KEntry e;
   if (k < a.Kred) {
     const int c = k % a.TC, t = k / a.TC;
@@ -128,15 +133,12 @@ __device__ __forceinline__ void write_ktab_entry(KEntry* __restrict__ tab, const
     e.off = 0;
     e.dhw = a.tapMask ? 31 : (-16384) & 0xffff;   // tap 31 / a row far above the image: never valid
   }
-  tab[k] = e;
+  return e;
 }
 
 // Forward: Wp[g][kq][i][j] = w[g*I + i][4*kq + j]  (w rows are Kred = Cg*R*S long, 0 beyond).
-// The first block of every k-quad also writes that quad's four table entries.
-__global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp, int I, int Ipad, int Kred, int KQ,
-                           KEntry* __restrict__ tab, KTabArgs ta) {
+__global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp, int I, int Ipad, int Kred, int KQ) {
   const int g = blockIdx.z, kq = blockIdx.y;
-  if (blockIdx.x == 0 && g == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= Ipad) return;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -151,14 +153,22 @@ __global__ void pack_w_fwd(const float* __restrict__ w, floatx4* __restrict__ wp
 
 // Input gradient, one stride-parity class: k = (ko*nTr + tr)*nTs + ts,
 // Wp[g][kq][c][j] = w[g*Kg + ko][c][r0 + tr*rstep][s0 + ts*sstep].
+// Up to kMaxMulti classes (the classes of one strided layer that have taps) are repacked by one
+// launch: blockIdx.z = class * groups + group, blockIdx.y runs to the longest class's KQ.
+constexpr int kMaxMulti = 4;
 struct PackDgrad {
   int Kg, Cg, R, S, Ipad, Kred, KQ;
   int nTr, nTs, r0, rstep, s0, sstep;
+  floatx4* wp;
 };
-__global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ wp, PackDgrad a,
-                             KEntry* __restrict__ tab, KTabArgs ta) {
-  const int g = blockIdx.z, kq = blockIdx.y;
-  if (blockIdx.x == 0 && g == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
+struct PackDgradMulti {
+  PackDgrad c[kMaxMulti];
+  int groups;
+};
+__global__ void pack_w_dgrad(const float* __restrict__ w, const PackDgradMulti m) {
+  const int cls = blockIdx.z / m.groups, g = blockIdx.z % m.groups, kq = blockIdx.y;
+  const PackDgrad& a = m.c[cls];
+  if (kq >= a.KQ) return;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= a.Ipad) return;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -173,7 +183,7 @@ __global__ void pack_w_dgrad(const float* __restrict__ w, floatx4* __restrict__ 
       }
     }
   }
-  wp[((size_t)g * a.KQ + kq) * a.Ipad + c] = floatx4{v[0], v[1], v[2], v[3]};
+  a.wp[((size_t)g * a.KQ + kq) * a.Ipad + c] = floatx4{v[0], v[1], v[2], v[3]};
 }
 
 // Dense input gradient: every stride-parity class becomes Cg rows of one GEMM over the union
@@ -185,15 +195,12 @@ struct PackDense {
   int Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, HxWx, Wx;
   int cellW;   // pixel classes per cell row (a multiple of sw)
 };
-__global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restrict__ wp, PackDense a,
-                                   KEntry* __restrict__ tab, KTabArgs ta, int4* __restrict__ rowtab) {
+__global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restrict__ wp, PackDense a) {
   const int kq = blockIdx.y;
-  if (blockIdx.x == 0 && threadIdx.x < 4) write_ktab_entry(tab, ta, 4 * kq + threadIdx.x);
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= a.Ipad) return;
   const int cls = i / a.Cg, c = i % a.Cg;
   const int ch = cls / a.cellW, cw = cls % a.cellW;
-  if (kq == 0 && i < a.I) rowtab[i] = make_int4(c * a.HxWx + ch * a.Wx + cw, ch, cw, c);
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if (i < a.I) {
 #pragma unroll
@@ -789,7 +796,6 @@ __global__ __launch_bounds__(kThreads, 3) void igemm_bf16(const Igemm p) {
 // Several data-parallel launches in one grid (the stride-parity classes of a strided input
 // gradient): blocks [first[i], first[i+1]) belong to launch i.  One grid instead of a short
 // launch per class, each with its own ramp-up and tail.
-constexpr int kMaxMulti = 4;
 struct IgemmMulti {
   Igemm c[kMaxMulti];
   int first[kMaxMulti + 1];
@@ -1047,33 +1053,191 @@ int launch_igemm_multi(IgemmMulti& m, int groups, TileChoice t, int prof_id) {
   return 0;
 }
 
-// Reduction-index tables depend only on the layer geometry: keep them across calls.
-struct KTabKey {
-  int v[11];
-  bool operator<(const KTabKey& o) const {
-    for (int i = 0; i < 11; ++i)
-      if (v[i] != o.v[i]) return v[i] < o.v[i];
-    return false;
-  }
+// ---- index tables ----------------------------------------------------------------------------------
+// Reduction-index tables (and the row tables of dense input gradients) depend only on the layer
+// geometry.  They are built on the host, checked there against the tensor they address, uploaded
+// once into a device buffer of their own and kept per geometry: nothing on the device ever writes
+// them, and they share no memory with the per-call workspace.  At kMaxTables geometries the cache
+// is dropped and rebuilt (after a stream sync); tt_empty_cache drops it too.
+constexpr size_t kMaxTables = 1024;
+struct DeviceTable {
+  void* dev = nullptr;
+  std::vector<char> host;   // stays alive while the upload may still be reading it
 };
-__global__ void build_ktab(KEntry* __restrict__ tab, KTabArgs a) {
-  const int k = blockIdx.x * blockDim.x + threadIdx.x;
-  if (k < a.Kpad) write_ktab_entry(tab, a, k);
+std::map<std::vector<int>, DeviceTable>& table_cache() {
+  static std::map<std::vector<int>, DeviceTable> cache;
+  return cache;
 }
-int cached_ktab(const KTabArgs& a, KEntry** out) {
-  static std::map<KTabKey, KEntry*> cache;
-  const KTabKey key{{a.Kred, a.Kpad, a.TB, a.TC, a.sa, a.sb, a.sc, a.stepH, a.stepW, a.tapMask, a.offBias}};
+int release_tables() {   // the caller has synchronised the stream
+  auto& cache = table_cache();
+  for (auto& kv : cache)
+    if (kv.second.dev) TT_HIP(hipFree(kv.second.dev));
+  cache.clear();
+  return 0;
+}
+// Looks `key` up; on a miss uploads `bytes` from `host` (already checked by the caller).
+int cached_table(const std::vector<int>& key, const void* host, size_t bytes, const void** out) {
+  auto& cache = table_cache();
   auto it = cache.find(key);
   if (it == cache.end()) {
-    TT_REQUIRE(cache.size() < 4096, "too many distinct convolution geometries for the table cache");
-    KEntry* tab = nullptr;
-    TT_HIP(hipMalloc((void**)&tab, sizeof(KEntry) * (size_t)a.Kpad));
-    build_ktab<<<ceil_div(a.Kpad, 256), 256, 0, tt::stream()>>>(tab, a);
-    TT_LAUNCH_CHECK();
-    it = cache.emplace(key, tab).first;
+    hipStream_t st = tt::stream();
+    if (cache.size() >= kMaxTables) {
+      TT_HIP(hipStreamSynchronize(st));
+      if (release_tables()) return -1;
+    }
+    DeviceTable t;
+    t.host.assign((const char*)host, (const char*)host + bytes);
+    TT_HIP(hipMalloc(&t.dev, bytes));
+    it = cache.emplace(key, std::move(t)).first;   // the vector's storage moves with it
+    hipError_t e = hipMemcpyAsync(it->second.dev, it->second.host.data(), bytes, hipMemcpyHostToDevice, st);
+    if (e != hipSuccess) {
+      (void)hipFree(it->second.dev);
+      cache.erase(it);
+      return tt::fail_hip(e, "hipMemcpyAsync(index table)", __FILE__, __LINE__);
+    }
   }
-  *out = it->second;
+  *out = it->second.dev;
   return 0;
+}
+
+// What the kernel will do with entry k of `tab` for launch `p`, replayed on the host for the
+// extreme pixels of every tap: wherever the kernel's own bounds rule calls a tap valid, the
+// element it would fetch must be the element (n, group, plane a, row, column) of the source
+// tensor that the reduction index stands for, and lie inside the tensor; padding entries must
+// never be valid; the 32-bit byte offsets of the buffer mode must stay in [0, 2^31).
+// `planes` = channels of the source per group, `src_elems` = elements of the whole source tensor.
+int check_ktab(const char* fn, const Igemm& p, const KTabArgs& ka, const std::vector<KEntry>& tab, int N, int groups,
+               int U, int V, int planes, long long src_elems) {
+  if (p.mode == kModeGemm) return 0;   // plain matrix product: no table is read
+  const bool mask = p.mode == kModeTapMask;
+  TT_REQUIRE((int)tab.size() == ka.Kpad && ka.Kpad % (4 * kBKQ) == 0 && ka.Kred <= ka.Kpad,
+             "%s: index table of %zu entries for a reduction of %d (%d padded)", fn, tab.size(), ka.Kred, ka.Kpad);
+  TT_REQUIRE(p.srcRow == p.Wlim && (long long)p.srcStrideG == (long long)planes * p.Hlim * p.Wlim &&
+                 (long long)N * p.srcStrideN <= src_elems,
+             "%s: source geometry of the launch does not describe an [N, C, %d, %d] tensor", fn, p.Hlim, p.Wlim);
+  TT_REQUIRE(!mask || ka.TB * ka.TC <= 31, "%s: %d x %d taps do not fit the 31-bit tap mask", fn, ka.TB, ka.TC);
+  const long long plane = (long long)p.Hlim * p.Wlim;
+  // images a 256-pixel tile can span beyond its first one (buffer offsets are relative to that)
+  const long long span = std::min<long long>(N - 1, 255 / ((long long)U * V) + 1);
+  for (int k = 0; k < ka.Kpad; ++k) {
+    const KEntry e = tab[k];
+    long long off;
+    int th, tw;
+    if (mask) {
+      const int tap = e.dhw;
+      if (k >= ka.Kred) {
+        TT_REQUIRE(tap == 31, "%s: padding entry %d of the index table names tap %d", fn, k, tap);
+        continue;
+      }
+      TT_REQUIRE(tap >= 0 && tap < ka.TB * ka.TC && e.off >= 0 && e.off % 4 == 0,
+                 "%s: index table entry %d: tap %d, byte offset %d", fn, k, tap, e.off);
+      off = e.off / 4 - ka.offBias;
+      th = (tap / ka.TC) * p.stepH;
+      tw = (tap % ka.TC) * p.stepW;
+    } else {
+      off = e.off;
+      th = (int)(short)(e.dhw & 0xffff);
+      tw = e.dhw >> 16;
+      if (k >= ka.Kred) {
+        TT_REQUIRE(th <= -16384, "%s: padding entry %d of the index table can be valid (row step %d)", fn, k, th);
+        continue;
+      }
+    }
+    const int a = k / (ka.TB * ka.TC), b = (k / ka.TC) % ka.TB, c = k % ka.TC;
+    TT_REQUIRE(th == b * p.stepH && tw == c * p.stepW, "%s: index table entry %d steps (%d, %d), tap (%d, %d)", fn, k, th,
+               tw, b, c);
+    // pixels u with 0 <= u*su + bh + th < Hlim, likewise v
+    auto range = [](int n, int stride, int base, int lim, int* lo, int* hi) {
+      *lo = base >= 0 ? 0 : (-base + stride - 1) / stride;
+      *hi = lim - 1 - base < 0 ? -1 : std::min(n - 1, (lim - 1 - base) / stride);
+    };
+    int ulo, uhi, vlo, vhi;
+    range(U, p.su, p.bh + th, p.Hlim, &ulo, &uhi);
+    range(V, p.sv, p.bw + tw, p.Wlim, &vlo, &vhi);
+    if (ulo > uhi || vlo > vhi) continue;   // no pixel uses this tap
+    TT_REQUIRE(a < planes, "%s: index table entry %d addresses plane %d of %d", fn, k, a, planes);
+    for (int iu = 0; iu < 2; ++iu)
+      for (int iv = 0; iv < 2; ++iv)
+        for (int in = 0; in < 2; ++in)
+          for (int ig = 0; ig < 2; ++ig) {
+            const long long u = iu ? uhi : ulo, v = iv ? vhi : vlo, n = in ? N - 1 : 0, g = ig ? groups - 1 : 0;
+            const long long ih0 = u * p.su + p.bh, iw0 = v * p.sv + p.bw;
+            const long long at = n * p.srcStrideN + g * p.srcStrideG + ih0 * p.srcRow + iw0 + off;
+            const long long want = n * p.srcStrideN + g * p.srcStrideG + a * plane + (ih0 + th) * p.srcRow + (iw0 + tw);
+            TT_REQUIRE(at == want && at >= 0 && at < src_elems,
+                       "%s: index table entry %d reaches element %lld of the source (expected %lld of %lld)", fn, k, at,
+                       want, src_elems);
+            if (mask) {
+              const long long lane = 4 * (std::min<long long>(n, span) * p.srcStrideN + ih0 * p.srcRow + iw0 + p.voffBias);
+              TT_REQUIRE(lane >= 0 && lane + e.off < (1LL << 31),
+                         "%s: index table entry %d: byte offset %lld + %d leaves the buffer range", fn, k, lane, e.off);
+            }
+          }
+  }
+  return 0;
+}
+
+// Set only inside tt_conv2d_check_tables_selftest (host-only checks): damages one entry of the
+// next tables built, to show that check_ktab refuses them.
+int g_selftest_fault_entry = -1, g_selftest_fault_delta = 0;
+
+// Builds the table for `ka`, checks it against launch `p`, and (unless `host_only`) returns the
+// device copy kept for this geometry.
+int make_ktab(const char* fn, const Igemm& p, const KTabArgs& ka, int N, int groups, int U, int V, int planes,
+              long long src_elems, bool host_only, const KEntry** out) {
+  if (p.mode == kModeGemm) {   // plain matrix product: the kernel reads no table
+    *out = nullptr;
+    return 0;
+  }
+  std::vector<int> key{0, ka.Kred, ka.Kpad, ka.TB, ka.TC, ka.sa, ka.sb, ka.sc, ka.stepH, ka.stepW, ka.tapMask, ka.offBias,
+                       p.mode, N, groups, U, V, planes, p.su, p.bh, p.sv, p.bw, p.Hlim, p.Wlim, p.voffBias};
+  if (!host_only) {
+    auto it = table_cache().find(key);
+    if (it != table_cache().end()) {   // checked when it was built
+      *out = (const KEntry*)it->second.dev;
+      return 0;
+    }
+  }
+  std::vector<KEntry> tab((size_t)ka.Kpad);
+  for (int k = 0; k < ka.Kpad; ++k) tab[(size_t)k] = ktab_entry(ka, k);
+  if (g_selftest_fault_entry >= 0 && g_selftest_fault_entry < ka.Kpad)   // tt_conv2d_check_tables_selftest only
+    tab[(size_t)g_selftest_fault_entry].off += g_selftest_fault_delta;
+  if (check_ktab(fn, p, ka, tab, N, groups, U, V, planes, src_elems)) return -1;
+  if (host_only) return 0;
+  return cached_table(key, tab.data(), sizeof(KEntry) * tab.size(), (const void**)out);
+}
+
+// Row table of a dense input gradient: GEMM row i = (pixel class (ch, cw) of the cell, channel c)
+// -> {element offset c*Hx*Wx + ch*Wx + cw inside an image, ch, cw, c}.  Checked: every row of
+// every cell that the kernel's bounds rule (oh + ch < Hx, ow + cw < Wx) lets through lands inside
+// the output tensor.
+int make_rowtab(const char* fn, int I, int Cg, int cellH, int cellW, int Hx, int Wx, int N, int U, int V,
+                bool host_only, const int4** out) {
+  std::vector<int> key{1, I, Cg, cellH, cellW, Hx, Wx, N, U, V};
+  if (!host_only) {
+    auto it = table_cache().find(key);
+    if (it != table_cache().end()) {
+      *out = (const int4*)it->second.dev;
+      return 0;
+    }
+  }
+  TT_REQUIRE(I == cellH * cellW * Cg, "%s: %d rows for a %d x %d cell of %d channels", fn, I, cellH, cellW, Cg);
+  std::vector<int4> tab((size_t)I);
+  const long long out_elems = (long long)N * Cg * Hx * Wx;
+  for (int i = 0; i < I; ++i) {
+    const int cls = i / Cg, c = i % Cg;
+    const int ch = cls / cellW, cw = cls % cellW;
+    tab[(size_t)i] = make_int4(c * Hx * Wx + ch * Wx + cw, ch, cw, c);
+    // last cell row / column that still holds this class, last image
+    const long long u = (Hx - 1 - ch) / cellH, v = (Wx - 1 - cw) / cellW;
+    if (Hx - 1 - ch < 0 || Wx - 1 - cw < 0) continue;
+    TT_REQUIRE(u < U && v < V, "%s: row table: class (%d, %d) needs cell (%lld, %lld) of %d x %d", fn, ch, cw, u, v, U, V);
+    const long long at = (long long)(N - 1) * Cg * Hx * Wx + (u * cellH) * Wx + v * cellW + tab[(size_t)i].x;
+    TT_REQUIRE(at >= 0 && at < out_elems && u * cellH + ch < Hx && v * cellW + cw < Wx,
+               "%s: row table entry %d reaches element %lld of %lld", fn, i, at, out_elems);
+  }
+  if (host_only) return 0;
+  return cached_table(key, tab.data(), sizeof(int4) * tab.size(), (const void**)out);
 }
 
 int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
@@ -1101,6 +1265,10 @@ int dense_cell_min_tiles() { return g_dense_cell_min_tiles >= 0 ? g_dense_cell_m
 
 }  // namespace
 
+namespace tt {
+int conv_release_tables() { return release_tables(); }
+}  // namespace tt
+
 extern "C" {
 
 int tt_set_conv_dense_cell_min_tiles(int tiles) {
@@ -1110,17 +1278,23 @@ int tt_set_conv_dense_cell_min_tiles(int tiles) {
 }
 
 // `size_only`: report the workspace bytes this call would ask the library for and do nothing else.
+// `check_only`: build and check every index table the call would use, on the host alone (no
+// device is touched, tensor pointers are not looked at).
 static int conv2d_fwd(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
-                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, size_t* size_only) {
-  TT_REQUIRE_INIT();
-  TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
-  TT_REQUIRE_ALIGNED("tt_conv2d_fwd_f32", x, w, y);
+                      int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, size_t* size_only,
+                      bool check_only = false) {
+  const char* fn = "tt_conv2d_fwd_f32";
+  if (!check_only) {
+    TT_REQUIRE_INIT();
+    TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
+    TT_REQUIRE_ALIGNED("tt_conv2d_fwd_f32", x, w, y);
+  }
   const int P = (H + 2 * ph - dh * (R - 1) - 1) / sh + 1;
   const int Q = (W + 2 * pw - dw * (S - 1) - 1) / sw + 1;
   TT_REQUIRE(H + 2 * ph - dh * (R - 1) - 1 >= 0 && W + 2 * pw - dw * (S - 1) - 1 >= 0,
              "tt_conv2d_fwd_f32: kernel (%d x %d, dilation %d x %d) larger than padded input (%d x %d)", R, S, dh, dw,
              H + 2 * ph, W + 2 * pw);
-  if (check_common("tt_conv2d_fwd_f32", N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+  if (check_common(fn, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
   const int Cg = C / groups, Kg = K / groups;
   const int Kred = Cg * R * S;
   const int M = N * P * Q;
@@ -1130,16 +1304,13 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
   const int Ipad = ceil_div(Kg, t.bm) * t.bm;
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
-  const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
   if (size_only) {
-    *size_only = wp_bytes + tab_bytes + sk_workspace_bytes();
+    *size_only = wp_bytes + sk_workspace_bytes();
     return 0;
   }
-  void* ws;
-  if (tt::workspace(wp_bytes + tab_bytes + sk_workspace_bytes(), &ws)) return -1;
+  void* ws = nullptr;
+  if (!check_only && tt::workspace(wp_bytes + sk_workspace_bytes(), &ws)) return -1;
   floatx4* wp = (floatx4*)ws;
-  KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
-  hipStream_t st = tt::stream();
   // weight rows that are a whole number of chunks long are k-major 16-byte quads already
   const bool in_place = Kred % (4 * kBKQ) == 0;
 
@@ -1162,35 +1333,37 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
   p.kStride = H * W;
   p.Kred = Kred;
   KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw, 0, 0};
-  choose_mode(p, ka, R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && (H * W) % 4 == 0, N, P, Q,
+  choose_mode(p, ka, plain && (H * W) % 4 == 0, N, P, Q,
               in_place ? (long long)sizeof(float) * K * Kred : (long long)wp_bytes);
-  {
+  if (make_ktab(fn, p, ka, N, groups, P, Q, Cg, (long long)N * C * H * W, check_only, &p.ktab)) return -1;
+  if (check_only) return 0;
+  if (!in_place) {
     tt::ProfScope prof(TT_PROF_CONV_PREP);
-    if (in_place) {
-      if (cached_ktab(ka, &tab)) return -1;
-    } else {
-      pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, Kg, Ipad, Kred, KQ, tab, ka);
-      TT_LAUNCH_CHECK();
-    }
+    pack_w_fwd<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, tt::stream()>>>(w, wp, Kg, Ipad, Kred, KQ);
+    TT_LAUNCH_CHECK();
   }
-  p.ktab = tab;
-  return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes + tab_bytes));
+  return launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_FWD, (floatx4*)((char*)ws + wp_bytes));
 }
 
 static int conv2d_dgrad(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
                         int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
-                        int Q, size_t* size_only) {
-  TT_REQUIRE_INIT();
-  TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
-  TT_REQUIRE_ALIGNED("tt_conv2d_dgrad_f32", dy, w, dx);
-  if (check_common("tt_conv2d_dgrad_f32", N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+                        int Q, size_t* size_only, bool check_only = false) {
+  const char* fn = "tt_conv2d_dgrad_f32";
+  if (!check_only) {
+    TT_REQUIRE_INIT();
+    TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
+    TT_REQUIRE_ALIGNED("tt_conv2d_dgrad_f32", dy, w, dx);
+  }
+  if (check_common(fn, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q)) return -1;
+  const long long dy_elems = (long long)N * K * P * Q;
   // One dy pixel per image spread over a whole R x S kernel (the first layer of a transposed
   // generator: latent vector -> R x S map): every dx pixel has exactly one tap, tap (h, w), so
   // dx[n][(c,h,w)] = sum_k dy[n][k] * w[k][(c,h,w)] is the input gradient of a 1x1 convolution
   // with C*R*S channels on 1x1 images.  As R x S taps it would run R*S times the products.
   if (P == 1 && Q == 1 && R * S > 1 && ph == 0 && pw == 0 && dh == 1 && dw == 1 && Hx == R && Wx == S && groups == 1 &&
       bias == nullptr && tt::fits_i32((long long)C * R * S))
-    return conv2d_dgrad(dy, w, nullptr, dx, N, C * R * S, 1, 1, K, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1, 1, size_only);
+    return conv2d_dgrad(dy, w, nullptr, dx, N, C * R * S, 1, 1, K, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1, 1, size_only,
+                        check_only);
   const int Cg = C / groups, Kg = K / groups;
   const int gh = gcd(sh, dh), gw = gcd(sw, dw);
   const int rstep = sh / gh, sstep = sw / gw;   // valid taps of a class: r0, r0+rstep, ...
@@ -1198,7 +1371,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
 
   const int classes = sh * sw;
   TT_REQUIRE(classes <= 4096, "tt_conv2d_dgrad_f32: stride %d x %d not supported", sh, sw);
-  hipStream_t st = tt::stream();
+  hipStream_t st = check_only ? nullptr : tt::stream();
 
   if (groups == 1 && classes > 1 && classes * Cg <= 64 && Hx >= sh && Wx >= sw) {
     // tiny Cg: per-class GEMMs would fill 3 of 32 MFMA rows; stack all classes as rows instead
@@ -1260,19 +1433,15 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       t.sk_blocks = 0;
       const int Ipad = t.bm;
       const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)KQ * Ipad, 256);
-      const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQ * 4, 256);
-      const size_t row_bytes = align_up(sizeof(int4) * (size_t)I, 256);
       if (size_only) {
-        *size_only = wp_bytes + tab_bytes + row_bytes;
+        *size_only = wp_bytes;
         return 0;
       }
-      void* ws;
-      if (tt::workspace(wp_bytes + tab_bytes + row_bytes, &ws)) return -1;
+      void* ws = nullptr;
+      if (!check_only && tt::workspace(wp_bytes, &ws)) return -1;
       floatx4* wp = (floatx4*)ws;
-      KEntry* tab = (KEntry*)((char*)ws + wp_bytes);
-      int4* rowtab = (int4*)((char*)ws + wp_bytes + tab_bytes);
       Igemm p{};
-      p.src = dy; p.wp = wp; p.wbuf = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.src = dy; p.wp = wp; p.wbuf = wp; p.bias = bias; p.out = dx;
       p.I = I; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
       p.divUV = tt::make_fastdiv((uint32_t)(U * V));
       p.divV = tt::make_fastdiv((uint32_t)V);
@@ -1281,13 +1450,19 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       p.srcStrideN = K * P * Q; p.srcStrideG = 0;
       p.outStrideN = C * Hx * Wx; p.outStrideG = 0; p.outStrideI = 0; p.outRow = Wx;
       p.ou = cellH; p.ouh = 0; p.ov = cellW; p.ovw = 0;
-      p.rowtab = rowtab; p.outH = Hx; p.outW = Wx;
+      p.outH = Hx; p.outW = Wx;
       KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1, 0, 0};
       choose_mode(p, ka, false, N, U, V, (long long)wp_bytes);
+      // (one group: the launch's group stride is 0, the check takes the whole of dy as one group)
+      Igemm pc = p;
+      pc.srcStrideG = K * P * Q;
+      if (make_ktab(fn, pc, ka, N, 1, U, V, Kg, dy_elems, check_only, &p.ktab)) return -1;
+      if (make_rowtab(fn, I, Cg, cellH, cellW, Hx, Wx, N, U, V, check_only, &p.rowtab)) return -1;
+      if (check_only) return 0;
       {
         tt::ProfScope prof(TT_PROF_CONV_PREP);
         PackDense pa{Kg, Cg, R, S, sh, sw, ph, pw, dh, dw, Na, Nb, amin, bmin, I, Ipad, Kred, KQ, Hx * Wx, Wx, cellW};
-        pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa, tab, ka, rowtab);
+        pack_w_dgrad_dense<<<dim3(ceil_div(Ipad, 64), KQ), 64, 0, st>>>(w, wp, pa);
         TT_LAUNCH_CHECK();
       }
       return launch_igemm(p, 1, t, TT_PROF_CONV_IGEMM_DGRAD, nullptr);
@@ -1299,14 +1474,13 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
   const int KQmax = ceil_div((long long)Kg * max_taps_r * max_taps_s, 4 * kBKQ) * kBKQ;
   const int IpadMax = ceil_div(Cg, 128) * 128;
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQmax * IpadMax, 256);
-  const size_t tab_bytes = align_up(sizeof(KEntry) * (size_t)KQmax * 4, 256);
   if (size_only) {
-    *size_only = (wp_bytes + tab_bytes) * classes + sk_workspace_bytes();
+    *size_only = wp_bytes * classes + sk_workspace_bytes();
     return 0;
   }
-  void* ws;
-  if (tt::workspace((wp_bytes + tab_bytes) * classes + sk_workspace_bytes(), &ws)) return -1;
-  floatx4* sk_partial = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * classes);
+  void* ws = nullptr;
+  if (!check_only && tt::workspace(wp_bytes * classes + sk_workspace_bytes(), &ws)) return -1;
+  floatx4* sk_partial = (floatx4*)((char*)ws + wp_bytes * classes);
 
   // Parity classes without a tap hold only bias (or zero).  Without a bias it is cheaper to
   // clear dx once with a streaming fill than to launch a strided store kernel per empty class.
@@ -1330,7 +1504,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       any_empty |= !has;
     }
     if (any_empty) {
-      TT_HIP(hipMemsetAsync(dx, 0, sizeof(float) * (size_t)N * C * Hx * Wx, st));
+      if (!check_only) TT_HIP(hipMemsetAsync(dx, 0, sizeof(float) * (size_t)N * C * Hx * Wx, st));
       prefilled = true;
     }
   }
@@ -1352,6 +1526,13 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
   TileChoice multi_tile{};
   bool multi_ok = !allow_stream_k && tap_rows * tap_cols <= kMaxMulti;
 
+  // First every class is planned (launch descriptor, index table, repack descriptor), then the
+  // repacks run, then the matrix products.
+  std::vector<PackDgradMulti> packs;
+  std::vector<int> pack_kq, pack_ipad;
+  int pack_n = 0;
+  const int pack_limit = groups * kMaxMulti <= 65535 ? kMaxMulti : 1;   // grid.z = classes * groups
+  std::vector<std::pair<Igemm, TileChoice>> singles;
   int slot = 0;
   for (int ch = 0; ch < sh && ch < Hx; ++ch) {
     // taps r with (ch + ph - r*dh) % sh == 0
@@ -1374,10 +1555,9 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k,
                                        (plain && KQ / kBKQ <= 32 && !bf16_math()) || !allow_stream_k);
       const int Ipad = ceil_div(Cg, t.bm) * t.bm;
-      floatx4* wp = (floatx4*)((char*)ws + (wp_bytes + tab_bytes) * slot);
-      KEntry* tab = (KEntry*)((char*)wp + wp_bytes);
+      floatx4* wp = (floatx4*)((char*)ws + wp_bytes * slot);
       Igemm p{};
-      p.src = dy; p.wp = wp; p.wbuf = wp; p.ktab = tab; p.bias = bias; p.out = dx;
+      p.src = dy; p.wp = wp; p.wbuf = wp; p.bias = bias; p.out = dx;
       p.I = Cg; p.Ipad = Ipad; p.KQ = KQ; p.M = M;
       p.divUV = tt::make_fastdiv((uint32_t)(U * V));
       p.divV = tt::make_fastdiv((uint32_t)V);
@@ -1399,18 +1579,22 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
         choose_mode(p, ka,
                     R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && Hx == P && Wx == Q && (P * Q) % 4 == 0,
                     N, U, V, in_place ? (long long)sizeof(float) * K * Cg : (long long)wp_bytes);
-        tt::ProfScope prof(TT_PROF_CONV_PREP);
+        if (make_ktab(fn, p, ka, N, groups, U, V, Kg, dy_elems, check_only, &p.ktab)) return -1;
         if (in_place && p.mode != kModeCompare) {
           p.wbuf = w;
           p.wTransStride = Cg;
-          if (p.mode == kModeTapMask) {
-            if (cached_ktab(ka, &tab)) return -1;
-            p.ktab = tab;
-          }
         } else {
-          PackDgrad pa{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep};
-          pack_w_dgrad<<<dim3(ceil_div(Ipad, 64), KQ, groups), 64, 0, st>>>(w, wp, pa, tab, ka);
-          TT_LAUNCH_CHECK();
+          // the classes' repacks are collected and launched together, kMaxMulti classes per launch
+          if (packs.empty() || pack_n == pack_limit) {
+            packs.push_back(PackDgradMulti{});
+            packs.back().groups = groups;
+            pack_n = 0;
+            pack_kq.push_back(0);
+            pack_ipad.push_back(0);
+          }
+          packs.back().c[pack_n++] = PackDgrad{Kg, Cg, R, S, Ipad, Kred, KQ, nTr, nTs, r0, rstep, s0, sstep, wp};
+          pack_kq.back() = KQ > pack_kq.back() ? KQ : pack_kq.back();
+          pack_ipad.back() = Ipad > pack_ipad.back() ? Ipad : pack_ipad.back();
         }
       }
       if (multi_ok && KQ > 0 && t.sk_blocks == 0 && p.wTransStride == 0 && p.mode != kModeGemm &&
@@ -1426,9 +1610,20 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
         multi_tile = t;
         continue;
       }
-      if (launch_igemm(p, groups, t, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
+      singles.push_back({p, t});
     }
   }
+  if (check_only) return 0;
+  if (!packs.empty()) {
+    tt::ProfScope prof(TT_PROF_CONV_PREP);
+    for (size_t i = 0; i < packs.size(); ++i) {
+      const int n = i + 1 < packs.size() ? pack_limit : pack_n;
+      pack_w_dgrad<<<dim3(ceil_div(pack_ipad[i], 64), pack_kq[i], groups * n), 64, 0, st>>>(w, packs[i]);
+      TT_LAUNCH_CHECK();
+    }
+  }
+  for (auto& one : singles)
+    if (launch_igemm(one.first, groups, one.second, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
   if (multi.n == 1) {
     if (launch_igemm(multi.c[0], groups, multi_tile, TT_PROF_CONV_IGEMM_DGRAD, sk_partial)) return -1;
   } else if (multi.n > 1) {
@@ -1446,6 +1641,47 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
                         int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
                         int Q) {
   return conv2d_dgrad(dy, w, bias, dx, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q, nullptr);
+}
+
+// Host-only: builds every index table the corresponding call would use for this geometry and checks
+// each entry's reach against the tensors, as the calls themselves do once per new geometry.
+int tt_conv2d_check_tables_fwd_f32(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
+                                   int dh, int dw, int groups) {
+  return conv2d_fwd(nullptr, nullptr, nullptr, nullptr, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr,
+                    true);
+}
+
+int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R, int S, int sh, int sw, int ph, int pw,
+                                     int dh, int dw, int groups, int P, int Q) {
+  return conv2d_dgrad(nullptr, nullptr, nullptr, nullptr, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q,
+                      nullptr, true);
+}
+
+// Host-only: damages single table entries of a few geometries (an offset one row, one element or
+// one image off, in both addressing modes, forward and input gradient) and returns 0 when the
+// table check refuses every damaged table and accepts the undamaged ones.
+int tt_conv2d_check_tables_selftest(void) {
+  struct Case { int R, pad, stride, entry, delta; };
+  // 3x3 pad 1 (tap-mask tables: byte offsets), 6x6 pad 2 (compare-mode tables: element offsets)
+  const Case cases[] = {{3, 1, 1, 0, 4}, {3, 1, 1, 5, 4 * 9}, {3, 1, 2, 17, -4 * 9 * 9}, {6, 2, 1, 3, 1}, {6, 2, 1, 40, -14}};
+  int bad = 0;
+  for (const Case& c : cases) {
+    const int H = 9 + c.R, P = (H + 2 * c.pad - c.R) / c.stride + 1;
+    for (int pass = 0; pass < 2; ++pass) {
+      for (int damaged = 0; damaged < 2; ++damaged) {
+        g_selftest_fault_entry = damaged ? c.entry : -1;
+        g_selftest_fault_delta = c.delta;
+        const int rc = pass == 0 ? conv2d_fwd(nullptr, nullptr, nullptr, nullptr, 3, 8, H, H, 16, c.R, c.R, c.stride, c.stride,
+                                              c.pad, c.pad, 1, 1, 1, nullptr, true)
+                                 : conv2d_dgrad(nullptr, nullptr, nullptr, nullptr, 3, 8, H, H, 16, c.R, c.R, c.stride,
+                                                c.stride, c.pad, c.pad, 1, 1, 1, P, P, nullptr, true);
+        g_selftest_fault_entry = -1;
+        if ((rc != 0) != (damaged != 0)) ++bad;
+      }
+    }
+  }
+  TT_REQUIRE(bad == 0, "tt_conv2d_check_tables_selftest: %d of 20 table checks gave the wrong verdict", bad);
+  return 0;
 }
 
 // The queries run the same argument checks and planning as the calls themselves, with placeholder

@@ -485,8 +485,12 @@ struct PixKey {
 // The pixel table depends only on the geometry: built on first use, kept for the process
 // (16 bytes per output pixel; at most kMaxPixTables geometries, then the oldest are dropped).
 constexpr size_t kMaxPixTables = 256;
-int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
+std::map<PixKey, int4*>& pixtab_cache() {
   static std::map<PixKey, int4*> cache;
+  return cache;
+}
+int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
+  auto& cache = pixtab_cache();
   const PixKey key{{N, P, Q, p.H, p.W, p.sh, p.sw, p.ph, p.pw, p.dh, p.dw, p.R, p.S, p.chunks}};
   auto it = cache.find(key);
   if (it == cache.end()) {
@@ -500,7 +504,10 @@ int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
     int4* tab = nullptr;
     TT_HIP(hipMalloc((void**)&tab, sizeof(int4) * (size_t)entries));
     wgrad_build_pixtab<<<ceil_div(entries, 256), 256, 0, st>>>(tab, p, entries, N);
-    TT_LAUNCH_CHECK();
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+      (void)hipFree(tab);
+      return tt::fail_hip(e, "wgrad_build_pixtab", __FILE__, __LINE__);
+    }
     it = cache.emplace(key, tab).first;
   }
   *out = it->second;
@@ -523,6 +530,15 @@ void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStre
 }
 
 }  // namespace
+
+namespace tt {
+int wgrad_release_tables() {   // the caller has synchronised the stream
+  auto& cache = pixtab_cache();
+  for (auto& kv : cache) TT_HIP(hipFree(kv.second));
+  cache.clear();
+  return 0;
+}
+}  // namespace tt
 
 extern "C" {
 

@@ -238,6 +238,7 @@ int tt_empty_cache(void) {
   if (s.ws) TT_HIP(hipFree(s.ws));
   s.ws = nullptr;
   s.ws_bytes = 0;
+  if (tt::conv_release_tables() || tt::wgrad_release_tables()) return -1;
   return 0;
 }
 

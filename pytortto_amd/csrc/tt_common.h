@@ -28,6 +28,11 @@ int workspace(size_t bytes, void** out);
 // `device`, which must be the current device (batchnorm.hip).  Called once per device by tt_init.
 int bn_scratch_init(int device);
 
+// Frees the per-geometry index tables of the convolution kernels (conv_igemm.hip) and the pixel
+// tables of the weight gradient (conv_wgrad.hip); the caller has synchronised the stream.
+int conv_release_tables();
+int wgrad_release_tables();
+
 // Brackets the launches made during its lifetime with events when profiling is enabled
 // (a negative kernel id switches it off for that scope).
 struct ProfScope {
