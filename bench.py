@@ -102,7 +102,7 @@ class BnLayer:
 
     def run_fwd(self, call):
         call('tt_bn_fwd_train_f32', self.x.ptr, self.gamma.ptr, self.beta.ptr, self.y.ptr, self.mean.ptr,
-             self.var.ptr, self.sd.ptr, self.rm.ptr, self.rv.ptr, self.rm.ptr, self.rv.ptr, 0.1, 1e-5, *self.dims)
+             self.var.ptr, self.sd.ptr, self.rm.ptr, self.rv.ptr, self.rm.ptr, self.rv.ptr, None, 0.1, 1e-5, *self.dims)
 
     def run_bwd(self, call):
         call('tt_bn_bwd_f32', self.x.ptr, self.dy.ptr, self.gamma.ptr, self.mean.ptr, self.var.ptr, self.sd.ptr,

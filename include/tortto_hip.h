@@ -16,7 +16,9 @@
  *     aligned); a misaligned pointer is refused with an error.  Exception: x and dy of
  *     tt_conv2d_wgrad_f32 may have any 4-byte alignment (it falls back to scalar fetches).
  *   - kernels are enqueued on one library-owned HIP stream and return immediately;
- *     tt_sync() / tt_memcpy_d2h() wait for them.  One caller thread at a time.
+ *     tt_sync() / tt_memcpy_d2h() wait for them.  Calls may come from several threads: one lock
+ *     inside the library serialises them (allocator, workspace and table caches are shared), and
+ *     work enqueued by different threads runs in the order the calls took the lock.
  *   - tensors are limited to 2^31-1 elements each (32-bit element offsets in the kernels);
  *     larger ones are rejected with an error.
  */
@@ -54,6 +56,9 @@ int tt_event_record(void* event);
 int tt_event_elapsed_ms(void* start, void* stop, float* ms);   /* waits for `stop` */
 int tt_event_destroy(void* event);
 
+/* ---- measurement instrumentation: per-kernel timing and calibration probes.  Used by bench.py
+ *      only; a binding of the convolution / BatchNorm path needs nothing from this section. ---- */
+
 /* Per-kernel timing (no counterpart in the reference).  While enabled, the library brackets
  * each launch of its main kernels with HIP events on its stream; tt_profile_read() waits for
  * the stream and returns the number of launches and their summed duration since
@@ -76,8 +81,8 @@ enum {
 int tt_profile_enable(int on);
 int tt_profile_read(int kernel_id, long long* launches, double* total_ms);
 
-/* Calibration probes (no counterpart in the reference): what the device sustains with nothing
- * else in the way.  tt_probe_mfma_f32 runs `launches` back-to-back launches (about 1.3 ms each)
+/* Calibration probes (no counterpart in the reference; measurement only): what the device sustains
+ * with nothing else in the way.  tt_probe_mfma_f32 runs `launches` back-to-back launches (about 1.3 ms each)
  * of dense v_mfma_f32_32x32x2_f32 with per-lane varying operands and reports TFLOP/s (host
  * pointers); tt_probe_hbm_f32 streams `bytes` (>= 64 MiB) with 16 KiB contiguous chunks per
  * block: read-only GB/s and copy GB/s (read + written bytes). */
@@ -167,11 +172,13 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW);
  *   if running_mean_in/var_in are not NULL:
  *     running_mean_out = (1-momentum)*running_mean_in + momentum*mean
  *     running_var_out  = (1-momentum)*running_var_in  + momentum*var*(M/(M-1)),  M = N*HW
- *   (in/out may alias).  Returns an error when M == 1 (grad_nn.py:899-904). */
+ *   (in/out may alias).  num_batches_tracked (one float, may be NULL) is incremented by one: the
+ *   module's `self.num_batches_tracked.data += 1` (nn/modules/batchnorm.py:66) without a launch of
+ *   its own.  Returns an error when M == 1 (grad_nn.py:899-904). */
 int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y,
                         float* save_mean, float* save_var_eps, float* save_sd,
                         const float* running_mean_in, const float* running_var_in,
-                        float* running_mean_out, float* running_var_out,
+                        float* running_mean_out, float* running_var_out, float* num_batches_tracked,
                         double momentum, double eps, int N, int C, int HW);
 
 /* tt_bn_fwd_train_f32 for callers that cannot allocate (code under HIP graph capture, tight
@@ -188,6 +195,7 @@ int tt_bn_fwd_train_noalloc_f32(const float* x, const float* gamma, const float*
                                 float* save_mean, float* save_var_eps, float* save_sd,
                                 const float* running_mean_in, const float* running_var_in,
                                 float* running_mean_out, float* running_var_out,
+                                float* num_batches_tracked,
                                 double momentum, double eps, int N, int C, int HW);
 
 /* Normalisation with given statistics (eval mode), autograd/grad_nn.py:931-959:
@@ -259,8 +267,10 @@ int tt_log_softmax_bwd_f32(const float* g, const float* y, float* dx, int R, int
  * weights or NULL; ignore_index acts only when >= 0, as in the reference (:301-305).
  * reduction: 0 none (out[R]), 1 sum, 2 mean (out[1]); `count` (device, 1 float) receives the
  * mean's divisor: R without weights, else the number of rows with non-zero weight (:315-319).
- * The backward takes the same `count`; g is [R] for reduction none, else one value.  Targets
- * outside [0, C) raise IndexError in the reference; here such rows contribute nothing. */
+ * The backward takes the same `count`; g is [R] for reduction none, else one value.  Targets in
+ * [-C, -1] count from the end, as the reference's NumPy indexing does; targets outside [-C, C)
+ * raise IndexError in the reference: a kernel cannot raise, so such a row's loss (and a summed or
+ * averaged loss with it) is NaN and its gradient row is zero. */
 int tt_nll_loss_fwd_f32(const float* logp, const long long* target, const float* weight, float* out,
                         float* count, int R, int C, long long ignore_index, int reduction);
 int tt_nll_loss_bwd_f32(const float* g, const long long* target, const float* weight, const float* count,

@@ -48,8 +48,8 @@ PROTOTYPES = {
     'tt_workspace_size_conv2d_dgrad_f32': [POINTER(c_size_t)] + [_I] * 16,
     'tt_workspace_size_conv2d_wgrad_f32': [POINTER(c_size_t)] + [_I] * 16,
     'tt_workspace_size_bn_f32': [POINTER(c_size_t), _I, _I, _I],
-    'tt_bn_fwd_train_f32': [_P] * 11 + [c_double, c_double, _I, _I, _I],
-    'tt_bn_fwd_train_noalloc_f32': [_P] * 11 + [c_double, c_double, _I, _I, _I],
+    'tt_bn_fwd_train_f32': [_P] * 12 + [c_double, c_double, _I, _I, _I],
+    'tt_bn_fwd_train_noalloc_f32': [_P] * 12 + [c_double, c_double, _I, _I, _I],
     'tt_bn_fwd_eval_f32': [_P] * 9 + [c_double, _I, _I, _I],
     'tt_bn_bwd_f32': [_P] * 9 + [_I, _I, _I],
     'tt_relu_fwd_f32': [_P, _P, c_size_t],

@@ -135,16 +135,23 @@ class BatchNorm(Function):
         beta = None if xt2 is None else xt2.data
         have_running = running_mean is not None and running_var is not None
         cshape = (xd0.shape[1],) + (1,) * (xd0.ndim - 2)
+        count_batch = params.get('count_batch')
         if training:
             _verify_batch_size(xd0.shape)
             yd0, mean, var_eps, sd, new_rm, new_rv = ops.bn_fwd_train(
                 xd0, gamma, beta, running_mean.data if have_running else None,
-                running_var.data if have_running else None, momentum, eps)
+                running_var.data if have_running else None, momentum, eps,
+                num_batches_tracked=None if count_batch is None else count_batch.data)
             if have_running:            # the buffers are re-bound to new arrays (grad_nn.py:929-930)
                 running_mean.data = new_rm
                 running_var.data = new_rv
         elif have_running:
             yd0, mean, var_eps, sd = ops.bn_fwd_eval(xd0, gamma, beta, running_mean.data, running_var.data, eps)
+        elif xd0.size == xd0.shape[1]:
+            # eval mode without buffers and one value per channel: the batch statistics are the value
+            # itself and zero (grad_nn.py:935-937); only training refuses this shape (:921-922)
+            yd0, mean, var_eps, sd = ops.bn_fwd_eval(xd0, gamma, beta, xd0.reshape((xd0.shape[1],)),
+                                                     hiparray(np.zeros(xd0.shape[1], np.float32)), eps)
         else:
             yd0, mean, var_eps, sd, _, _ = ops.bn_fwd_train(xd0, gamma, beta, None, None, 0.0, eps)
         yt0 = build_links(yd0, grad_fn=ctx)

@@ -383,6 +383,7 @@ struct FwdArgs {
   const double2* partial;
   int partial_splits;       // partials per channel written by the first sweep
   float one_minus_mom, mom, unbias, eps;
+  float* nbt;               // training: the module's batch counter, incremented by one (may be null)
 };
 
 // kMode: 0 planes, 1 flat VEC=4, 2 flat VEC=1
@@ -424,6 +425,7 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_apply(FwdArgs a, Geometry g) 
           a.rv_out[c] =
               __fadd_rn(__fmul_rn(a.one_minus_mom, a.rv_in[c]), __fmul_rn(a.mom, __fmul_rn(var, a.unbias)));
         }
+        if (a.nbt && c == 0) *a.nbt = __fadd_rn(*a.nbt, 1.0f);   // one thread of the whole grid
       }
     }
   }
@@ -535,6 +537,7 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) 
       a.rm_out[c] = __fadd_rn(__fmul_rn(a.one_minus_mom, a.rm_in[c]), __fmul_rn(a.mom, mean));
       a.rv_out[c] = __fadd_rn(__fmul_rn(a.one_minus_mom, a.rv_in[c]), __fmul_rn(a.mom, __fmul_rn(var, a.unbias)));
     }
+    if (a.nbt && c == 0) *a.nbt = __fadd_rn(*a.nbt, 1.0f);
   }
   __syncthreads();
   const Coef k = sk;
@@ -713,8 +716,8 @@ extern "C" {
 static int bn_fwd_train(const char* fn, const float* x, const float* gamma, const float* beta, float* y,
                         float* save_mean, float* save_var_eps, float* save_sd, const float* running_mean_in,
                         const float* running_var_in, float* running_mean_out, float* running_var_out,
-                        double momentum, double eps, int N, int C, int HW, double2* fixed_partials,
-                        size_t fixed_capacity) {
+                        float* num_batches_tracked, double momentum, double eps, int N, int C, int HW,
+                        double2* fixed_partials, size_t fixed_capacity) {
   TT_REQUIRE_INIT();
   if (check_shape(fn, N, C, HW)) return -1;
   TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
@@ -731,6 +734,7 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
   a.rm_in = track ? running_mean_in : nullptr; a.rv_in = track ? running_var_in : nullptr;
   a.rm_out = running_mean_out; a.rv_out = running_var_out;
   a.given_mean = nullptr; a.given_var = nullptr;
+  a.nbt = num_batches_tracked;
   a.one_minus_mom = (float)(1.0 - momentum);
   a.mom = (float)momentum;
   a.unbias = (float)((double)m / (double)(m - 1));
@@ -781,23 +785,24 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
 int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
                         float* save_var_eps, float* save_sd, const float* running_mean_in,
                         const float* running_var_in, float* running_mean_out, float* running_var_out,
-                        double momentum, double eps, int N, int C, int HW) {
+                        float* num_batches_tracked, double momentum, double eps, int N, int C, int HW) {
   return bn_fwd_train("tt_bn_fwd_train_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd, running_mean_in,
-                      running_var_in, running_mean_out, running_var_out, momentum, eps, N, C, HW, nullptr, 0);
+                      running_var_in, running_mean_out, running_var_out, num_batches_tracked, momentum, eps, N, C, HW,
+                      nullptr, 0);
 }
 
 int tt_bn_fwd_train_noalloc_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
                                 float* save_var_eps, float* save_sd, const float* running_mean_in,
                                 const float* running_var_in, float* running_mean_out, float* running_var_out,
-                                double momentum, double eps, int N, int C, int HW) {
+                                float* num_batches_tracked, double momentum, double eps, int N, int C, int HW) {
   TT_REQUIRE_INIT();
   int dev = -1;
   TT_HIP(hipGetDevice(&dev));
   TT_REQUIRE(dev >= 0 && dev < kMaxDevices && g_scratch_ptr[dev] != nullptr,
              "tt_bn_fwd_train_noalloc_f32: the scratch array of device %d was not set up by tt_init", dev);
   return bn_fwd_train("tt_bn_fwd_train_noalloc_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd,
-                      running_mean_in, running_var_in, running_mean_out, running_var_out, momentum, eps, N, C, HW,
-                      g_scratch_ptr[dev], (size_t)kScratchPartials);
+                      running_mean_in, running_var_in, running_mean_out, running_var_out, num_batches_tracked, momentum,
+                      eps, N, C, HW, g_scratch_ptr[dev], (size_t)kScratchPartials);
 }
 
 int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, float* y, const float* mean,

@@ -1272,6 +1272,7 @@ int conv_release_tables() { return release_tables(); }
 extern "C" {
 
 int tt_set_conv_dense_cell_min_tiles(int tiles) {
+  TT_API_LOCK();
   TT_REQUIRE(tiles >= 0 && tiles <= (1 << 20), "tt_set_conv_dense_cell_min_tiles: %d is out of range (0..2^20)", tiles);
   g_dense_cell_min_tiles = tiles;
   return 0;
@@ -1284,6 +1285,7 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
                       int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, size_t* size_only,
                       bool check_only = false) {
   const char* fn = "tt_conv2d_fwd_f32";
+  TT_API_LOCK();
   if (!check_only) {
     TT_REQUIRE_INIT();
     TT_REQUIRE(x && w && y, "tt_conv2d_fwd_f32: null tensor pointer");
@@ -1349,6 +1351,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
                         int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
                         int Q, size_t* size_only, bool check_only = false) {
   const char* fn = "tt_conv2d_dgrad_f32";
+  TT_API_LOCK();
   if (!check_only) {
     TT_REQUIRE_INIT();
     TT_REQUIRE(dy && w && dx, "tt_conv2d_dgrad_f32: null tensor pointer");
@@ -1661,6 +1664,7 @@ int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R,
 // one image off, in both addressing modes, forward and input gradient) and returns 0 when the
 // table check refuses every damaged table and accepts the undamaged ones.
 int tt_conv2d_check_tables_selftest(void) {
+  TT_API_LOCK();
   struct Case { int R, pad, stride, entry, delta; };
   // 3x3 pad 1 (tap-mask tables: byte offsets), 6x6 pad 2 (compare-mode tables: element offsets)
   const Case cases[] = {{3, 1, 1, 0, 4}, {3, 1, 1, 5, 4 * 9}, {3, 1, 2, 17, -4 * 9 * 9}, {6, 2, 1, 3, 1}, {6, 2, 1, 40, -14}};

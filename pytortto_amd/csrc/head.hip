@@ -118,15 +118,18 @@ __global__ __launch_bounds__(kThreads) void nll_loss_fwd(const float* __restrict
   const bool weighted = weight != nullptr || ignore_index >= 0;
   double s = 0.0, cnt = 0.0;
   for (int n = threadIdx.x; n < R; n += kThreads) {
-    const long long t = target[n];
+    const long long t0 = target[n];
+    const long long t = t0 < 0 ? t0 + C : t0;      // -C..-1 count from the end, as NumPy indexing does (:300, :309)
     float w = 1.f, v = 0.f;
     if (t >= 0 && t < C) {
       if (weight) w = weight[t];
       v = -logp[(size_t)n * C + t];
     } else {
-      w = 0.f;                                     // out-of-range class: contributes nothing
+      // a class outside [-C, C): the reference's indexing raises IndexError; a kernel cannot raise,
+      // so the row's loss -- and with it a summed or averaged loss -- becomes NaN
+      v = __builtin_nanf("");
     }
-    if (ignore_index >= 0 && t == ignore_index) w = 0.f;
+    if (ignore_index >= 0 && t0 == ignore_index) w = 0.f;
     if (weighted) v = v * w;
     if (reduction == 0) out[n] = v;
     s += (double)v;
@@ -164,11 +167,12 @@ __global__ __launch_bounds__(kThreads) void nll_loss_bwd(const float* __restrict
   for (size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x; e < total; e += stride) {
     const uint32_t n = tt::fd_div((uint32_t)e, divC);
     const long long c = (long long)((uint32_t)e - n * (uint32_t)C);
-    const long long t = target[n];
+    const long long t0 = target[n];
+    const long long t = t0 < 0 ? t0 + C : t0;      // negative classes count from the end, as in the forward
     float v = 0.f;
     if (c == t) {
       float w = weight ? weight[t] : 1.f;
-      if (ignore_index >= 0 && t == ignore_index) w = 0.f;
+      if (ignore_index >= 0 && t0 == ignore_index) w = 0.f;
       float gv = reduction == 0 ? g[n] : g[0];
       if (reduction == 2) gv = __fdiv_rn(gv, div);
       v = -gv * w;

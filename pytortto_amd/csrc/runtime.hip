@@ -79,6 +79,11 @@ int fail_hip(hipError_t e, const char* what, const char* file, int line) {
   return (int)e;
 }
 
+std::recursive_mutex& api_mutex() {
+  static std::recursive_mutex m;
+  return m;
+}
+
 hipStream_t stream() { return S().stream; }
 int compute_units() { return S().compute_units; }
 int conv_math() { return S().conv_math; }
@@ -154,6 +159,7 @@ extern "C" {
 const char* tt_last_error(void) { return g_err; }
 
 int tt_init(int device) {
+  TT_API_LOCK();
   State& s = S();
   if (s.ready) {
     TT_REQUIRE(device == s.device, "tt_init(%d): library already initialised on device %d", device, s.device);
@@ -281,12 +287,14 @@ int tt_memset(void* dst_dev, int byte_value, size_t bytes) {
 }
 
 int tt_set_conv_math(int mode) {
+  TT_API_LOCK();
   TT_REQUIRE(mode == TT_CONV_MATH_F32 || mode == TT_CONV_MATH_BF16, "tt_set_conv_math: unknown mode %d", mode);
   S().conv_math = mode;
   return 0;
 }
 
 int tt_get_conv_math(int* mode) {
+  TT_API_LOCK();
   TT_REQUIRE(mode != nullptr, "tt_get_conv_math: null output pointer");
   *mode = S().conv_math;
   return 0;

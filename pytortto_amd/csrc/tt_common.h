@@ -4,6 +4,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/tortto_hip.h"
 
 namespace tt {
@@ -11,6 +13,14 @@ namespace tt {
 // Records a message for tt_last_error() and returns a non-zero status.
 int fail(int code, const char* fmt, ...);
 int fail_hip(hipError_t e, const char* what, const char* file, int line);
+
+// One lock serialises the C ABI: the allocator's maps, the workspace, the table caches and the
+// profiling state are shared, and callers such as a Python process (ctypes releases the GIL
+// during a call; a device array may be finalised on another thread) reach them from several
+// threads.  Every entry point that touches that state holds the lock for its duration (calls only
+// enqueue work, so it is held for microseconds; tt_sync and the synchronous copies hold it while
+// they wait).  Recursive: entry points call each other.
+std::recursive_mutex& api_mutex();
 
 // The one stream every kernel of the library is enqueued on.
 hipStream_t stream();
@@ -93,6 +103,12 @@ inline bool all_aligned16(P... ptrs) { return (aligned16(ptrs) && ...); }
 #define TT_REQUIRE_ALIGNED(fn, ...) \
   TT_REQUIRE(tt::all_aligned16(__VA_ARGS__), "%s: tensor pointers must be 16-byte aligned", fn)
 
-#define TT_REQUIRE_INIT() TT_REQUIRE(tt::initialised(), "tt_init() has not been called")
+#define TT_CAT2(a, b) a##b
+#define TT_CAT(a, b) TT_CAT2(a, b)
+#define TT_API_LOCK() std::lock_guard<std::recursive_mutex> TT_CAT(tt_api_lock_, __LINE__)(tt::api_mutex())
+// Takes the API lock for the rest of the enclosing scope and refuses calls before tt_init().
+#define TT_REQUIRE_INIT() \
+  TT_API_LOCK();          \
+  TT_REQUIRE(tt::initialised(), "tt_init() has not been called")
 
 #define TT_LAUNCH_CHECK() TT_HIP(hipGetLastError())

@@ -52,16 +52,22 @@ class _BatchNorm(Module):
     def forward(self, inpt):
         self._check_input_dim(inpt)
         factor = None                                   # weight of the new batch in the running statistics
+        count_batch = None
         if self.training and self.track_running_stats:
-            self.num_batches_tracked.data += 1          # (:66)
-            factor = self.momentum if self.momentum is not None else 1.0 / self.num_batches_tracked.item()
+            if self.momentum is not None and self.num_batches_tracked.is_cuda and inpt.is_cuda:
+                # the counter's `+= 1` (:66) rides along in the training kernel; nothing reads it before
+                count_batch = self.num_batches_tracked
+                factor = self.momentum
+            else:
+                self.num_batches_tracked.data += 1      # (:66)
+                factor = self.momentum if self.momentum is not None else 1.0 / self.num_batches_tracked.item()
         # batch statistics are used in training mode, and in eval mode when there are no buffers (:75-78)
         no_buffers = self.running_mean is None and self.running_var is None
         batch_stats = self.training or no_buffers
         pass_buffers = self.track_running_stats or not self.training
         return F.batch_norm(inpt, self.running_mean if pass_buffers else None,
                             self.running_var if pass_buffers else None, self.weight, self.bias, batch_stats,
-                            factor, self.eps)
+                            factor, self.eps, _count_batch=count_batch)
 
 
 class BatchNorm1d(_BatchNorm):

@@ -90,10 +90,12 @@ def _nchw(x):
     return n, c, x.size // (n * c) if n * c else 0
 
 
-def bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps):
+def bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None):
     """Training forward (autograd/grad_nn.py:921-930, :942-959).  Returns
     ``(y, mean, var_eps, sd, new_running_mean, new_running_var)``; the last two are new arrays
-    (``None`` without running statistics), as the reference rebinds ``.data``."""
+    (``None`` without running statistics), as the reference rebinds ``.data``.
+    ``num_batches_tracked`` (a one-element device array) is incremented by one in the same launch:
+    the module's ``num_batches_tracked.data += 1`` (nn/modules/batchnorm.py:66)."""
     _f32(x, gamma, beta, running_mean, running_var)
     n, c, hw = _nchw(x)
     y = hiparray.empty(x.shape)
@@ -103,7 +105,8 @@ def bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps):
     new_rv = hiparray.empty((c,)) if track else None
     _hip.call('tt_bn_fwd_train_f32', x.ptr, _ptr(gamma), _ptr(beta), y.ptr, mean.ptr, var_eps.ptr, sd.ptr,
               _ptr(running_mean) if track else None, _ptr(running_var) if track else None,
-              _ptr(new_rm), _ptr(new_rv), float(momentum if momentum is not None else 0.0), float(eps), n, c, hw)
+              _ptr(new_rm), _ptr(new_rv), _ptr(num_batches_tracked),
+              float(momentum if momentum is not None else 0.0), float(eps), n, c, hw)
     return y, mean, var_eps, sd, new_rm, new_rv
 
 

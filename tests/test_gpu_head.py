@@ -98,6 +98,38 @@ def test_nll_loss(reduction, weighted, ignore_index):
                                                               count), rtol=1e-6, atol=1e-8)
 
 
+@pytest.mark.parametrize('weighted', [False, True])
+def test_nll_loss_negative_and_out_of_range_targets(weighted):
+    """Classes -C..-1 count from the end, as the reference's NumPy indexing does (grad_nn.py:300,
+    :306-309).  Classes outside [-C, C) raise IndexError there; on the device the loss turns NaN."""
+    from pytortto_amd import ops
+    rng = np.random.default_rng(8)
+    n, c = 40, 7
+    logp = oracle.log_softmax_forward(rng.standard_normal((n, c)).astype(np.float32))
+    target = rng.integers(-c, c, n)
+    assert (target < 0).any()
+    weight = rng.uniform(0.5, 2.0, c).astype(np.float32) if weighted else None
+    wd = None if weight is None else _dev(weight)
+    for reduction in ('mean', 'sum', 'none'):
+        loss, count = oracle.nll_loss_forward(logp, target, weight, 2, reduction)
+        td = _dev(target.astype(np.int64))
+        out, cnt = ops.nll_loss_fwd(_dev(logp), td, wd, 2, reduction)
+        np.testing.assert_allclose(out.get(), loss, rtol=1e-5, atol=1e-6)
+        g = rng.standard_normal(np.shape(loss)).astype(np.float32) if reduction == 'none' else np.float32(0.7)
+        grad = ops.nll_loss_bwd(_dev(np.asarray(g, np.float32)), logp.shape, td, wd, cnt, 2, reduction).get()
+        np.testing.assert_allclose(grad, oracle.nll_loss_backward(g, logp.shape, target, weight, 2, reduction, count),
+                                   rtol=1e-6, atol=1e-8)
+    for bad in (c, -c - 1, 1000):
+        with pytest.raises(IndexError):
+            oracle.nll_loss_forward(logp, np.where(np.arange(n) == 5, bad, target % c), weight, -100, 'mean')
+        td = _dev(np.where(np.arange(n) == 5, bad, target % c).astype(np.int64))
+        out, _ = ops.nll_loss_fwd(_dev(logp), td, wd, -100, 'mean')
+        assert np.isnan(out.get()).all()
+        rows, _ = ops.nll_loss_fwd(_dev(logp), td, wd, -100, 'none')
+        rows = rows.get()
+        assert np.isnan(rows[5]) and not np.isnan(np.delete(rows, 5)).any()
+
+
 def test_linear_log_softmax_nll_modules_on_device():
     """The head of the reference's ResNet examples: mean over (H, W), flatten, Linear, LogSoftmax,
     NLLLoss -- same graph (MeanBackward, ViewBackward, TransposeBackward, MmBackward, AddBackward)."""

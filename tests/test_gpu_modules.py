@@ -363,3 +363,25 @@ def test_add_backward_gives_each_operand_its_own_gradient_array():
     (at + at).backward(tt.tensor(g).cuda())
     assert np.array_equal(bt.grad.get(), g)
     assert np.array_equal(at.grad.get(), g + (g + g))
+
+
+def test_batch_norm_without_buffers_accepts_one_value_per_channel_outside_training():
+    """Only training refuses one value per channel (grad_nn.py:921-922); `F.batch_norm` with
+    training=False and no running buffers takes the batch statistics, here the value itself and
+    zero (:935-937), so y = beta.  (Through the module this shape is refused in eval mode too: it
+    passes training=True when it has no buffers, nn/modules/batchnorm.py:75-78.)"""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    gamma = np.arange(1, 6, dtype=np.float32)
+    beta = np.linspace(-1, 1, 5).astype(np.float32)
+    x = np.random.randn(1, 5, 1, 1).astype(np.float32)
+    bn = nn.BatchNorm2d(5, track_running_stats=False)
+    bn.cuda()
+    for mode in (bn.train, bn.eval):
+        mode()
+        with pytest.raises(ValueError, match='Expected more than 1 value per channel'):
+            bn(tt.tensor(x).cuda())
+    y = nn.functional.batch_norm(tt.tensor(x).cuda(), None, None, tt.tensor(gamma).cuda(), tt.tensor(beta).cuda(),
+                                 False, 0.1, 1e-5).cpu().detach().numpy()
+    y_ref, _, _, _ = oracle.batch_norm_forward(x, gamma, beta, None, None, False, 0.1, 1e-5)
+    np.testing.assert_allclose(y, y_ref, rtol=1e-6, atol=1e-7)

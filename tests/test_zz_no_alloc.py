@@ -29,8 +29,10 @@ def _run(entry, x, gamma, beta, rm0, rv0):
     rmd, rvd = hiparray(rm0), hiparray(rv0)
     y = hiparray.empty(x.shape)
     outs = [hiparray.empty((c,)) for _ in range(5)]   # mean, var+eps, sd, running mean, running var
+    counter = hiparray(np.array([7.0], np.float32))   # num_batches_tracked: incremented by the call
     _hip.call(entry, xd.ptr, gd.ptr, bd.ptr, y.ptr, outs[0].ptr, outs[1].ptr, outs[2].ptr, rmd.ptr, rvd.ptr,
-              outs[3].ptr, outs[4].ptr, 0.1, 1e-5, n, c, hw)
+              outs[3].ptr, outs[4].ptr, counter.ptr, 0.1, 1e-5, n, c, hw)
+    assert counter.get()[0] == 8.0
     return [y.get()] + [o.get() for o in outs]
 
 
@@ -85,4 +87,4 @@ def test_noalloc_entry_rejects_sizes_beyond_the_scratch_array():
     dummy = hiparray.empty((16,))
     with pytest.raises(RuntimeError, match='fixed scratch array'):
         _hip.call('tt_bn_fwd_train_noalloc_f32', dummy.ptr, None, None, dummy.ptr, dummy.ptr, dummy.ptr, dummy.ptr,
-                  None, None, None, None, 0.1, 1e-5, 64, 2049, 4096)
+                  None, None, None, None, None, 0.1, 1e-5, 64, 2049, 4096)
