@@ -19,8 +19,14 @@
  *     tt_sync() / tt_memcpy_d2h() wait for them.  Calls may come from several threads: one lock
  *     inside the library serialises them (allocator, workspace and table caches are shared), and
  *     work enqueued by different threads runs in the order the calls took the lock.
- *   - tensors are limited to 2^31-1 elements each (32-bit element offsets in the kernels);
- *     larger ones are rejected with an error.
+ *   - tensor sizes: the convolution kernels index with 32-bit element offsets, so one image
+ *     ([C, H, W] resp. [K, P, Q]) and the weights must each stay below 2^31 elements; a batch
+ *     whose tensors have 2^31 elements or more is cut into runs of images inside the library
+ *     (forward, input gradient: one set of launches per run; weight gradient: one set of partial
+ *     sums per run, added by the one reduce kernel).  BatchNorm and the elementwise kernels use
+ *     64-bit offsets; BatchNorm needs a channel's N*HW values and an image's C*HW below 2^31.
+ *     Pooling, the classifier head and the spatial extents (< 16384) keep 32-bit limits and
+ *     reject what exceeds them.
  */
 #ifndef TORTTO_HIP_H
 #define TORTTO_HIP_H

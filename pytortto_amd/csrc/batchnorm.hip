@@ -637,8 +637,11 @@ int plan(int N, int C, int HW, Geometry* g, int* mode) {
 
 int check_shape(const char* fn, int N, int C, int HW) {
   TT_REQUIRE(N > 0 && C > 0 && HW > 0, "%s: N, C, HW must be positive (got %d, %d, %d)", fn, N, C, HW);
-  TT_REQUIRE(tt::fits_i32((long long)N * C * HW), "%s: tensor of %lld elements exceeds 2^31-1", fn,
-             (long long)N * C * HW);
+  // element offsets are 64-bit; what must fit 32 bits are a channel's N*HW values (the index the
+  // blocks split) and one image's C*HW
+  TT_REQUIRE(tt::fits_i32((long long)N * HW) && tt::fits_i32((long long)C * HW),
+             "%s: a channel (%lld values) or an image (%lld) exceeds 2^31-1 elements", fn, (long long)N * HW,
+             (long long)C * HW);
   TT_REQUIRE(C <= 65535, "%s: more than 65535 channels are not supported", fn);
   return 0;
 }

@@ -1252,7 +1252,7 @@ int check_common(const char* fn, int N, int C, int H, int W, int K, int R, int S
              "%s: spatial extents must stay below 16384", fn);
   TT_REQUIRE(tt::fits_i32((long long)N * C * H * W) && tt::fits_i32((long long)N * K * P * Q) &&
                  tt::fits_i32((long long)K * (C / groups) * R * S),
-             "%s: a tensor exceeds 2^31-1 elements", fn);
+             "%s: one image or the weights exceed 2^31-1 elements", fn);
   return 0;
 }
 
@@ -1635,27 +1635,60 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
   return 0;
 }
 
+// The kernels index with 32-bit element offsets.  Forward and input gradient are independent per
+// image, so a batch whose tensors have 2^31 elements or more runs as several calls over runs of
+// images that stay below that (one image and the weights must fit on their own).
+static int images_per_call(int N, long long image_a, long long image_b) {
+  const long long image = image_a > image_b ? image_a : image_b;
+  if (N <= 0 || image <= 0 || (long long)N * image < 2147483647LL) return N;
+  const long long per = 2147483646LL / image;
+  return (int)(per < 1 ? 1 : per);
+}
+static long long out_size(long long in, int k, int s, int p, int d) { return (in + 2LL * p - (long long)d * (k - 1) - 1) / s + 1; }
+
 int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
                       int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
-  return conv2d_fwd(x, w, bias, y, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr);
+  const long long xi = (long long)C * H * W;
+  const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
+  const int per = images_per_call(N, xi, yi);
+  if (per >= N) return conv2d_fwd(x, w, bias, y, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr);
+  for (int n0 = 0; n0 < N; n0 += per) {
+    const int n = N - n0 < per ? N - n0 : per;
+    if (int rc = conv2d_fwd(x + (size_t)n0 * xi, w, bias, y + (size_t)n0 * yi, n, C, H, W, K, R, S, sh, sw, ph, pw, dh,
+                            dw, groups, nullptr))
+      return rc;
+  }
+  return 0;
 }
 
 int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
                         int K, int R, int S, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P,
                         int Q) {
-  return conv2d_dgrad(dy, w, bias, dx, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q, nullptr);
+  const long long xi = (long long)C * Hx * Wx, yi = (long long)K * P * Q;
+  const int per = images_per_call(N, xi, yi);
+  if (per >= N) return conv2d_dgrad(dy, w, bias, dx, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q, nullptr);
+  for (int n0 = 0; n0 < N; n0 += per) {
+    const int n = N - n0 < per ? N - n0 : per;
+    if (int rc = conv2d_dgrad(dy + (size_t)n0 * yi, w, bias, dx + (size_t)n0 * xi, n, C, Hx, Wx, K, R, S, sh, sw, ph, pw,
+                              dh, dw, groups, P, Q, nullptr))
+      return rc;
+  }
+  return 0;
 }
 
 // Host-only: builds every index table the corresponding call would use for this geometry and checks
 // each entry's reach against the tensors, as the calls themselves do once per new geometry.
 int tt_conv2d_check_tables_fwd_f32(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
                                    int dh, int dw, int groups) {
+  const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
+  N = images_per_call(N, (long long)C * H * W, yi);
   return conv2d_fwd(nullptr, nullptr, nullptr, nullptr, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr,
                     true);
 }
 
 int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R, int S, int sh, int sw, int ph, int pw,
                                      int dh, int dw, int groups, int P, int Q) {
+  N = images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q);
   return conv2d_dgrad(nullptr, nullptr, nullptr, nullptr, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q,
                       nullptr, true);
 }
@@ -1694,6 +1727,8 @@ int tt_workspace_size_conv2d_fwd_f32(size_t* bytes, int N, int C, int H, int W, 
                                      int ph, int pw, int dh, int dw, int groups) {
   TT_REQUIRE(bytes, "tt_workspace_size_conv2d_fwd_f32: null result pointer");
   const float* in = reinterpret_cast<const float*>(uintptr_t(256));
+  const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
+  N = images_per_call(N, (long long)C * H * W, yi);   // the largest of the calls a long batch is cut into
   return conv2d_fwd(in, in, nullptr, const_cast<float*>(in), N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups,
                     bytes);
 }
@@ -1702,6 +1737,7 @@ int tt_workspace_size_conv2d_dgrad_f32(size_t* bytes, int N, int C, int Hx, int 
                                        int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q) {
   TT_REQUIRE(bytes, "tt_workspace_size_conv2d_dgrad_f32: null result pointer");
   const float* in = reinterpret_cast<const float*>(uintptr_t(256));
+  N = images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q);
   return conv2d_dgrad(in, in, nullptr, const_cast<float*>(in), N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups,
                       P, Q, bytes);
 }

@@ -20,7 +20,9 @@
 // masked when the values are written to LDS.  Offsets are relative to the first image of the
 // chunk; geometries whose offsets could reach 2 GiB, or with more than 31 taps, take the
 // compare-and-select path instead.
+#include <algorithm>
 #include <map>
+#include <vector>
 
 #include "tt_common.h"
 
@@ -553,13 +555,15 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
   TT_REQUIRE(sh > 0 && sw > 0 && dh > 0 && dw_ > 0 && ph >= 0 && pw >= 0, "%s: stride/dilation must be positive, padding non-negative", fn);
   TT_REQUIRE(groups > 0 && groups <= 65535 && C % groups == 0 && K % groups == 0, "%s: channels (%d, %d) not divisible by groups=%d", fn, C, K, groups);
   TT_REQUIRE(H + 2 * ph + R * dh < 16384 && W + 2 * pw + S * dw_ < 16384, "%s: spatial extents must stay below 16384", fn);
-  TT_REQUIRE(tt::fits_i32((long long)N * C * H * W) && tt::fits_i32((long long)N * K * P * Q) &&
-                 tt::fits_i32((long long)K * (C / groups) * R * S),
-             "%s: a tensor exceeds 2^31-1 elements", fn);
+  // The kernels index with 32-bit element offsets.  A batch whose tensors have 2^31 elements or
+  // more is cut into runs of images that stay below that; every run writes its own partial sums
+  // and the reduce kernel adds the partials of all runs, still in a fixed order.
+  const long long image = std::max((long long)C * H * W, (long long)K * P * Q);
+  TT_REQUIRE(tt::fits_i32(image) && tt::fits_i32((long long)K * (C / groups) * R * S),
+             "%s: one image or the weights exceed 2^31-1 elements", fn);
+  const int per_run = (int)std::min<long long>(N, std::max<long long>(1, 2147483646LL / image));
   const int Cg = C / groups, Kg = K / groups;
   const int J = Cg * R * S;
-  const long long Mll = (long long)N * P * Q;
-  const int M = (int)Mll;
 
   int bm = 128, bn = 128;
   if (Kg <= 64) bm = 64;
@@ -571,78 +575,93 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
   if (R == 1 && S == 1 && Kg >= 128) bn = 64;
   const int tilesI = ceil_div(Kg, bm), tilesJ = ceil_div(J, bn);
   const long long tiles = (long long)tilesI * tilesJ * groups;
-  const int chunks = ceil_div(M, kBK);
   // Two blocks fit a CU (LDS), so 2 x CUs (512 on an MI355X) run at a time and all take equally
   // long: fill one such round as well as possible, or two rounds if that fills them clearly better;
   // at least 8 chunks (256 pixels) of work per split.
   const int kSlots = 2 * tt::compute_units();
-  int splits = (int)(kSlots / tiles);
-  const int two = (int)(2 * kSlots / tiles);
-  if ((double)tiles * two / (2.0 * kSlots) > (double)tiles * splits / kSlots + 0.08) splits = two;
-  if (splits > chunks / 8) splits = chunks / 8;
-  if (splits < 1) splits = 1;
-  if (splits > 4096) splits = 4096;
-  int cps = ceil_div(chunks, splits);
-  splits = ceil_div(chunks, cps);
+  struct Run { int n0, n, chunks, cps, splits, slot0; };
+  std::vector<Run> runs;
+  int slots = 0;
+  for (int n0 = 0; n0 < N; n0 += per_run) {
+    Run r{};
+    r.n0 = n0;
+    r.n = std::min(per_run, N - n0);
+    r.chunks = ceil_div((long long)r.n * P * Q, kBK);
+    int splits = (int)(kSlots / tiles);
+    const int two = (int)(2 * kSlots / tiles);
+    if ((double)tiles * two / (2.0 * kSlots) > (double)tiles * splits / kSlots + 0.08) splits = two;
+    if (splits > r.chunks / 8) splits = r.chunks / 8;
+    if (splits < 1) splits = 1;
+    if (splits > 4096) splits = 4096;
+    r.cps = ceil_div(r.chunks, splits);
+    r.splits = ceil_div(r.chunks, r.cps);
+    r.slot0 = slots;
+    slots += r.splits;
+    runs.push_back(r);
+  }
 
   const size_t elems = (size_t)groups * Kg * J;
   if (size_only) {
-    *size_only = splits > 1 ? sizeof(float) * elems * splits : 0;
+    *size_only = slots > 1 ? sizeof(float) * elems * slots : 0;
     return 0;
   }
   float* target = dw;
-  if (splits > 1) {
+  if (slots > 1) {
     void* ws;
-    if (tt::workspace(sizeof(float) * elems * splits, &ws)) return -1;
+    if (tt::workspace(sizeof(float) * elems * slots, &ws)) return -1;
     target = (float*)ws;
   }
-  Wgrad p{};
-  p.x = x; p.dy = dy; p.out = target;
-  p.Kg = Kg; p.J = J; p.M = M;
-  p.chunks = chunks; p.chunksPerSplit = cps;
-  p.divPQ = tt::make_fastdiv((uint32_t)(P * Q));
-  p.divQ = tt::make_fastdiv((uint32_t)Q);
-  p.divRS = tt::make_fastdiv((uint32_t)(R * S));
-  p.divS = tt::make_fastdiv((uint32_t)S);
-  p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw; p.dh = dh; p.dw = dw_;
-  p.H = H; p.W = W; p.HW = H * W;
-  p.xStrideN = C * H * W; p.xStrideG = Cg * H * W;
-  p.dyStrideN = K * P * Q; p.dyStrideG = Kg * P * Q;
-  p.PQ = P * Q;
-  p.tilesI = tilesI;
-  p.outStrideSplit = elems;
-  p.R = R; p.S = S;
-  p.xBias = ph * W + pw;
-  p.divDh = tt::make_fastdiv((uint32_t)dh);
-  p.divDw = tt::make_fastdiv((uint32_t)dw_);
-  if (R * S <= 31)
-    for (int r = 0; r < R; ++r) p.rowOnes |= 1u << (r * S);
-  // buffer path: byte offsets relative to the first image of a 32-pixel chunk stay below 2 GiB
-  // (a chunk spans at most 33 images; x offsets also carry the column's tap and channel offset)
-  const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
-                               ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
-  const bool buf = R * S <= 31 && reach < (1LL << 31) - (1LL << 20);
-  if (buf && cached_pixtab(p, N, P, Q, &p.pixtab)) return -1;
-  // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
-  const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)dy & 15) == 0;
-  const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)x & 15) == 0;
-  dim3 grid(tilesI * tilesJ, groups, splits);
   hipStream_t st = tt::stream();
-  {
-    tt::ProfScope prof(TT_PROF_CONV_WGRAD);
-    if (bm == 128 && bn == 128)
-      launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, st);
-    else if (bm == 64 && bn == 128)
-      launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, st);
-    else if (bm == 128 && bn == 64)
-      launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, st);
-    else
-      launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, st);
+  for (const Run& r : runs) {
+    Wgrad p{};
+    p.x = x + (size_t)r.n0 * C * H * W;
+    p.dy = dy + (size_t)r.n0 * K * P * Q;
+    p.out = target + (size_t)r.slot0 * elems;
+    p.Kg = Kg; p.J = J; p.M = r.n * P * Q;
+    p.chunks = r.chunks; p.chunksPerSplit = r.cps;
+    p.divPQ = tt::make_fastdiv((uint32_t)(P * Q));
+    p.divQ = tt::make_fastdiv((uint32_t)Q);
+    p.divRS = tt::make_fastdiv((uint32_t)(R * S));
+    p.divS = tt::make_fastdiv((uint32_t)S);
+    p.sh = sh; p.sw = sw; p.ph = ph; p.pw = pw; p.dh = dh; p.dw = dw_;
+    p.H = H; p.W = W; p.HW = H * W;
+    p.xStrideN = C * H * W; p.xStrideG = Cg * H * W;
+    p.dyStrideN = K * P * Q; p.dyStrideG = Kg * P * Q;
+    p.PQ = P * Q;
+    p.tilesI = tilesI;
+    p.outStrideSplit = elems;
+    p.R = R; p.S = S;
+    p.xBias = ph * W + pw;
+    p.divDh = tt::make_fastdiv((uint32_t)dh);
+    p.divDw = tt::make_fastdiv((uint32_t)dw_);
+    if (R * S <= 31)
+      for (int rr = 0; rr < R; ++rr) p.rowOnes |= 1u << (rr * S);
+    // buffer path: byte offsets relative to the first image of a 32-pixel chunk stay below 2 GiB
+    // (a chunk spans at most 33 images; x offsets also carry the column's tap and channel offset)
+    const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
+                                 ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
+    const bool buf = R * S <= 31 && reach < (1LL << 31) - (1LL << 20);
+    if (buf && cached_pixtab(p, r.n, P, Q, &p.pixtab)) return -1;
+    // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
+    const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)p.dy & 15) == 0;
+    const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)p.x & 15) == 0;
+    dim3 grid(tilesI * tilesJ, groups, r.splits);
+    {
+      tt::ProfScope prof(TT_PROF_CONV_WGRAD);
+      if (bm == 128 && bn == 128)
+        launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, st);
+      else if (bm == 64 && bn == 128)
+        launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, st);
+      else if (bm == 128 && bn == 64)
+        launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, st);
+      else
+        launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, st);
+    }
+    TT_LAUNCH_CHECK();
   }
-  TT_LAUNCH_CHECK();
-  if (splits > 1) {
+  if (slots > 1) {
     tt::ProfScope prof(TT_PROF_CONV_WGRAD_REDUCE);
-    wgrad_reduce<<<ceil_div((long long)elems, 256), kThreads, 0, st>>>(target, dw, elems, splits);
+    wgrad_reduce<<<ceil_div((long long)elems, 256), kThreads, 0, st>>>(target, dw, elems, slots);
     TT_LAUNCH_CHECK();
   }
   return 0;
