@@ -218,6 +218,23 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma,
                   const float* save_mean, const float* save_var_eps, const float* save_sd,
                   float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
 
+/* BatchNorm followed by ReLU in one pass each way (no single counterpart in the reference, which
+ * runs BatchNorm, autograd/grad_nn.py:921-959 and :966-989, and Relu, :56-67, as separate array
+ * expressions; the two autograd nodes stay separate on the host side).
+ * tt_bn_relu_fwd_train_f32: tt_bn_fwd_train_f32 whose output is y = maximum(bn(x), 0), NaN kept;
+ * the normalised values themselves are not stored (the backward pass needs x and the statistics,
+ * the ReLU's backward its own output).
+ * tt_bn_relu_bwd_f32: tt_bn_bwd_f32 on the gradient g = dy * (relu_y > 0), formed as dy is read in
+ * both sweeps instead of by a kernel of its own; relu_y is the output of the forward call. */
+int tt_bn_relu_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y,
+                             float* save_mean, float* save_var_eps, float* save_sd,
+                             const float* running_mean_in, const float* running_var_in,
+                             float* running_mean_out, float* running_var_out, float* num_batches_tracked,
+                             double momentum, double eps, int N, int C, int HW);
+int tt_bn_relu_bwd_f32(const float* x, const float* dy, const float* relu_y, const float* gamma,
+                       const float* save_mean, const float* save_var_eps, const float* save_sd,
+                       float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
+
 /* ---- workspace queries (no counterpart in the reference) -------------------------------------- */
 
 /* Bytes of library workspace (repacked weights, index tables, partial sums) the corresponding call

@@ -50,6 +50,8 @@ PROTOTYPES = {
     'tt_workspace_size_bn_f32': [POINTER(c_size_t), _I, _I, _I],
     'tt_bn_fwd_train_f32': [_P] * 12 + [c_double, c_double, _I, _I, _I],
     'tt_bn_fwd_train_noalloc_f32': [_P] * 12 + [c_double, c_double, _I, _I, _I],
+    'tt_bn_relu_fwd_train_f32': [_P] * 12 + [c_double, c_double, _I, _I, _I],
+    'tt_bn_relu_bwd_f32': [_P] * 10 + [_I, _I, _I],
     'tt_bn_fwd_eval_f32': [_P] * 9 + [c_double, _I, _I, _I],
     'tt_bn_bwd_f32': [_P] * 9 + [_I, _I, _I],
     'tt_relu_fwd_f32': [_P, _P, c_size_t],
@@ -114,8 +116,44 @@ def lib():
     return handle
 
 
+# ---- one deferred operation ----------------------------------------------------------------------
+# An operation whose result the very next operation may absorb (BatchNorm's normalisation into a
+# following ReLU, a ReLU's gradient mask into the BatchNorm backward behind it) is not launched at
+# once: its caller parks it here.  The next operation either takes it over (``take_pending`` and a
+# fused launch) or, like any other call into the library, finds it run first -- ``call`` flushes
+# before it does anything else, so a deferred operation never outlives the next library call and
+# nothing can read or overwrite its operands in between.
+_pending = None
+
+
+def defer(op):
+    """Park ``op`` (an object with ``run()``); whatever was parked before runs now."""
+    global _pending
+    flush()
+    _pending = op
+
+
+def pending():
+    return _pending
+
+
+def take_pending():
+    global _pending
+    op, _pending = _pending, None
+    return op
+
+
+def flush():
+    op = take_pending()
+    if op is not None:
+        op.run()
+
+
 def call(name, *args):
-    """Call ``name`` through the C ABI and raise ``RuntimeError(tt_last_error())`` on failure."""
+    """Call ``name`` through the C ABI and raise ``RuntimeError(tt_last_error())`` on failure.
+    A deferred operation runs first."""
+    if _pending is not None:
+        flush()
     check(getattr(lib(), name)(*args))
 
 

@@ -12,7 +12,7 @@ from math import prod
 
 import numpy as np
 
-from .. import ops
+from .. import _hip, ops
 from ..xparray import hiparray
 from .function import Function
 from .helper import build_links, inplace_precheck, inplace_update
@@ -138,7 +138,9 @@ class BatchNorm(Function):
         count_batch = params.get('count_batch')
         if training:
             _verify_batch_size(xd0.shape)
-            yd0, mean, var_eps, sd, new_rm, new_rv = ops.bn_fwd_train(
+            # the launch is parked: a ReLU that comes next absorbs it (one pass over the tensor
+            # instead of two), anything else triggers it as it is
+            yd0, mean, var_eps, sd, new_rm, new_rv = ops.bn_fwd_train_deferred(
                 xd0, gamma, beta, running_mean.data if have_running else None,
                 running_var.data if have_running else None, momentum, eps,
                 num_batches_tracked=None if count_batch is None else count_batch.data)
@@ -165,6 +167,13 @@ class BatchNorm(Function):
         gd0, = grad_outputs
         xd0, xd1 = ctx.saved_tensors
         p = ctx.params
+        parked = _hip.pending()
+        if parked.__class__ is ops.DeferredReluBackward and parked.out._buf is gd0._buf:
+            # the gradient comes straight from a ReLU whose mask has not been applied yet: apply it
+            # while reading dy (grad_nn.py:67 folded into :977-988)
+            _hip.take_pending()
+            return ops.bn_relu_bwd(xd0, parked.dy, parked.y, xd1, p['mean'], p['var'], p['sd'],
+                                   need=ctx.needs_input_grad)
         grad0, grad1, grad2 = ops.bn_bwd(xd0, gd0, xd1, p['mean'], p['var'], p['sd'], need=ctx.needs_input_grad)
         return grad0, grad1, grad2
 
@@ -175,7 +184,18 @@ class Relu(Function):
         xt0, = inputs
         xd0 = xt0.data
         inplace = params['inplace']
-        if xd0.__class__ is hiparray:
+        parked = _hip.pending()
+        if parked.__class__ is ops.DeferredBatchNorm and parked.y._buf is xd0._buf:
+            # the input is a BatchNorm output that has not been launched yet: one kernel writes
+            # maximum(bn(x), 0) directly (grad_nn.py:942-959 and :56 in one pass)
+            if inplace:
+                inplace_precheck(xt0)
+                _hip.take_pending().run_with_relu()
+                yt0 = inplace_update(xt0, ctx)
+            else:
+                yt0 = build_links(_hip.take_pending().run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
+            ctx.params['after_batch_norm'] = True
+        elif xd0.__class__ is hiparray:
             if inplace:
                 inplace_precheck(xt0)
                 ops.relu_fwd(xd0, out=xd0)
@@ -196,6 +216,9 @@ class Relu(Function):
         gd0, = grad_outputs
         yd0, = ctx.saved_tensors
         if yd0.__class__ is hiparray:
+            if ctx.params.get('after_batch_norm') and gd0.__class__ is hiparray:
+                # the BatchNorm backward that follows can apply the mask itself; parked until then
+                return ops.relu_bwd_deferred(gd0, yd0)
             return ops.relu_bwd(gd0, yd0)
         return gd0 * (yd0 > 0)
 

@@ -100,6 +100,16 @@ __device__ __forceinline__ void store_stream(float4* p, const float4 o) {
   __builtin_nontemporal_store(v, reinterpret_cast<fx4*>(p));
 }
 
+// ReLU fused behind the normalisation (tt_bn_relu_*): forward y = max(bn(x), 0) keeping NaN, as
+// NumPy's maximum does (autograd/grad_nn.py:56); backward g = dy * (y > 0) as a product (:67), so
+// that a non-finite dy at a masked element gives NaN like the unfused pair of kernels.
+__device__ __forceinline__ float relu1(float v) { return (v > 0.f || v != v) ? v : 0.f; }
+__device__ __forceinline__ float4 relu4(float4 v) { return make_float4(relu1(v.x), relu1(v.y), relu1(v.z), relu1(v.w)); }
+__device__ __forceinline__ float mask1(float g, float y) { return g * (y > 0.f ? 1.f : 0.f); }
+__device__ __forceinline__ float4 mask4(float4 g, float4 y) {
+  return make_float4(mask1(g.x, y.x), mask1(g.y, y.y), mask1(g.z, y.z), mask1(g.w, y.w));
+}
+
 constexpr int kStreamU = 8;   // float4 loads in flight per thread in the stream reduce kernel
 
 struct Geometry {
@@ -174,11 +184,12 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_planes(const float* __rest
 // vectors (flattened over planes, so no batch is cut short at a plane end) and issues kU loads
 // per tensor and thread before it consumes the first: enough bytes in flight per block that the
 // reduction tails of other blocks do not leave the memory system idle.
-template <int kKind>
+template <int kKind, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_reduce_stream(const float* __restrict__ x,
                                                              const float* __restrict__ dy,
                                                              const float* __restrict__ mean,
-                                                             double2* __restrict__ partial, Geometry g) {
+                                                             double2* __restrict__ partial, Geometry g,
+                                                             const float* __restrict__ ry = nullptr) {
   __shared__ double lds[2 * kWaves];
   const int c = blockIdx.y, split = blockIdx.x;
   constexpr bool kBwd = kKind == 1;
@@ -205,7 +216,8 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_stream(const float* __rest
       if constexpr (kBwd) {
         // dy is streamed in both backward sweeps: x is read four times per training pass, dy twice,
         // and at these sizes the memory-side cache cannot hold both
-        const float4 q = load_stream(reinterpret_cast<const float4*>(dy + off));
+        float4 q = load_stream(reinterpret_cast<const float4*>(dy + off));
+        if constexpr (kRelu) q = mask4(q, load_stream(reinterpret_cast<const float4*>(ry + off)));
         gq[u] = ok ? q : zero;
       }
     }
@@ -234,11 +246,12 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_stream(const float* __rest
 }
 
 // Flat kernel: any HW.  Vector index e over the channel's N*HW/VEC vectors, n = e / (HW/VEC).
-template <int kKind, int VEC>
+template <int kKind, int VEC, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_reduce_flat(const float* __restrict__ x,
                                                            const float* __restrict__ dy,
                                                            const float* __restrict__ mean,
-                                                           double2* __restrict__ partial, Geometry g) {
+                                                           double2* __restrict__ partial, Geometry g,
+                                                           const float* __restrict__ ry = nullptr) {
   __shared__ double lds[2 * kWaves];
   const int c = blockIdx.y, split = blockIdx.x;
   const uint32_t hwv = (uint32_t)g.HW / VEC;
@@ -257,12 +270,13 @@ __global__ __launch_bounds__(kThreads) void bn_reduce_flat(const float* __restri
       const float4 t = *reinterpret_cast<const float4*>(x + off);
       v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
       if constexpr (kBwd) {
-        const float4 u = *reinterpret_cast<const float4*>(dy + off);
+        float4 u = *reinterpret_cast<const float4*>(dy + off);
+        if constexpr (kRelu) u = mask4(u, *reinterpret_cast<const float4*>(ry + off));
         gq[0] = u.x; gq[1] = u.y; gq[2] = u.z; gq[3] = u.w;
       }
     } else {
       v[0] = x[off];
-      if constexpr (kBwd) gq[0] = dy[off];
+      if constexpr (kBwd) gq[0] = kRelu ? mask1(dy[off], ry[off]) : dy[off];
     }
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -303,10 +317,10 @@ __device__ __forceinline__ float4 apply4(const float4 v, const float4 gq, const 
   return o;
 }
 
-template <bool kBwd>
+template <bool kBwd, bool kRelu>
 __device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const float* __restrict__ dy,
                                               float* __restrict__ out, const Geometry& g, int c, int split,
-                                              const Coef k) {
+                                              const Coef k, const float* __restrict__ ry) {
   const int hw4 = g.HW >> 2;
   const int n0 = split * g.per_block;
   const int n1 = min(g.N, n0 + g.per_block);
@@ -316,6 +330,7 @@ __device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const
     const float4* __restrict__ px = reinterpret_cast<const float4*>(x + off);
     const float4* __restrict__ pg = reinterpret_cast<const float4*>(dy + (kBwd ? off : 0));
     float4* __restrict__ po = reinterpret_cast<float4*>(out + off);
+    const float4* __restrict__ pr = reinterpret_cast<const float4*>(ry + (kBwd && kRelu ? off : 0));
     for (int i0 = threadIdx.x; i0 < hw4; i0 += kThreads * kU) {
       float4 v[kU], gq[kU];
 #pragma unroll
@@ -324,22 +339,24 @@ __device__ __forceinline__ void sweep2_planes(const float* __restrict__ x, const
         // backward: the last use of x and dy in the pass; forward: x is read again by the backward
         v[u] = kBwd ? load_stream(px + i) : px[i];
         gq[u] = kBwd ? load_stream(pg + i) : v[u];
+        if constexpr (kBwd && kRelu) gq[u] = mask4(gq[u], load_stream(pr + i));
       }
 #pragma unroll
       for (int u = 0; u < kU; ++u) {
         const int i = i0 + kThreads * u;
         if (i < hw4) {
-          store_stream(po + i, apply4<kBwd>(v[u], gq[u], k));
+          const float4 o = apply4<kBwd>(v[u], gq[u], k);
+          store_stream(po + i, (!kBwd && kRelu) ? relu4(o) : o);
         }
       }
     }
   }
 }
 
-template <bool kBwd, int VEC>
+template <bool kBwd, int VEC, bool kRelu>
 __device__ __forceinline__ void sweep2_flat(const float* __restrict__ x, const float* __restrict__ dy,
                                             float* __restrict__ out, const Geometry& g, int c, int split,
-                                            const Coef k) {
+                                            const Coef k, const float* __restrict__ ry) {
   const uint32_t hwv = (uint32_t)g.HW / VEC;
   const uint32_t total = (uint32_t)g.N * hwv;
   const uint32_t e0 = (uint32_t)split * (uint32_t)g.per_block;
@@ -353,14 +370,20 @@ __device__ __forceinline__ void sweep2_flat(const float* __restrict__ x, const f
       const float4 v = kBwd ? load_stream(px) : *px;
       float4 gq = v;
       if (kBwd) gq = load_stream(reinterpret_cast<const float4*>(dy + off));
-      store_stream(reinterpret_cast<float4*>(out + off), apply4<kBwd>(v, gq, k));
+      if constexpr (kBwd && kRelu) gq = mask4(gq, load_stream(reinterpret_cast<const float4*>(ry + off)));
+      const float4 o = apply4<kBwd>(v, gq, k);
+      store_stream(reinterpret_cast<float4*>(out + off), (!kBwd && kRelu) ? relu4(o) : o);
     } else {
       const float v = kBwd ? __builtin_nontemporal_load(x + off) : x[off];
       float o;
-      if (kBwd)
-        o = fmaf(__builtin_nontemporal_load(dy + off), k.k1, fmaf(v - k.m, k.k2, k.k0));
-      else
+      if (kBwd) {
+        float gv = __builtin_nontemporal_load(dy + off);
+        if constexpr (kRelu) gv = mask1(gv, __builtin_nontemporal_load(ry + off));
+        o = fmaf(gv, k.k1, fmaf(v - k.m, k.k2, k.k0));
+      } else {
         o = fmaf(v - k.m, k.k1, k.k0);
+        if constexpr (kRelu) o = relu1(o);
+      }
       __builtin_nontemporal_store(o, out + off);
     }
   }
@@ -387,7 +410,7 @@ struct FwdArgs {
 };
 
 // kMode: 0 planes, 1 flat VEC=4, 2 flat VEC=1
-template <int kMode>
+template <int kMode, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_fwd_apply(FwdArgs a, Geometry g) {
   __shared__ Coef sk;
   const int c = g.C - 1 - (int)blockIdx.y;
@@ -431,9 +454,9 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_apply(FwdArgs a, Geometry g) 
   }
   __syncthreads();
   const Coef k = sk;
-  if (kMode == 0) sweep2_planes<false>(a.x, a.x, a.y, g, c, split, k);
-  if (kMode == 1) sweep2_flat<false, 4>(a.x, a.x, a.y, g, c, split, k);
-  if (kMode == 2) sweep2_flat<false, 1>(a.x, a.x, a.y, g, c, split, k);
+  if (kMode == 0) sweep2_planes<false, kRelu>(a.x, a.x, a.y, g, c, split, k, a.x);
+  if (kMode == 1) sweep2_flat<false, 4, kRelu>(a.x, a.x, a.y, g, c, split, k, a.x);
+  if (kMode == 2) sweep2_flat<false, 1, kRelu>(a.x, a.x, a.y, g, c, split, k, a.x);
 }
 
 struct BwdArgs {
@@ -448,9 +471,10 @@ struct BwdArgs {
   float* dbeta;
   const double2* partial;
   int partial_splits;
+  const float* ry;   // fused ReLU backward: the ReLU's output; dy is masked by (ry > 0) on the fly
 };
 
-template <int kMode>
+template <int kMode, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) {
   __shared__ Coef sk;
   const int c = g.C - 1 - (int)blockIdx.y;
@@ -476,9 +500,9 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) 
   if (a.dx == nullptr) return;
   __syncthreads();
   const Coef k = sk;
-  if (kMode == 0) sweep2_planes<true>(a.x, a.dy, a.dx, g, c, split, k);
-  if (kMode == 1) sweep2_flat<true, 4>(a.x, a.dy, a.dx, g, c, split, k);
-  if (kMode == 2) sweep2_flat<true, 1>(a.x, a.dy, a.dx, g, c, split, k);
+  if (kMode == 0) sweep2_planes<true, kRelu>(a.x, a.dy, a.dx, g, c, split, k, a.ry);
+  if (kMode == 1) sweep2_flat<true, 4, kRelu>(a.x, a.dy, a.dx, g, c, split, k, a.ry);
+  if (kMode == 2) sweep2_flat<true, 1, kRelu>(a.x, a.dy, a.dx, g, c, split, k, a.ry);
 }
 
 // ---- small channels: one kernel per pass ---------------------------------------------------------
@@ -502,7 +526,7 @@ __device__ __forceinline__ void for_channel_elements(const Geometry& g, F&& f) {
   }
 }
 
-template <int EMAX>
+template <int EMAX, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) {
   __shared__ double red[2 * kWaves];
   __shared__ Coef sk;
@@ -542,11 +566,12 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) 
   __syncthreads();
   const Coef k = sk;
   for_channel_elements<EMAX>(g, [&](int kk, size_t off) {
-    __builtin_nontemporal_store(fmaf(v[kk] - k.m, k.k1, k.k0), yc + off);
+    const float o = fmaf(v[kk] - k.m, k.k1, k.k0);
+    __builtin_nontemporal_store(kRelu ? relu1(o) : o, yc + off);
   });
 }
 
-template <int EMAX>
+template <int EMAX, bool kRelu = false>
 __global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) {
   __shared__ double red[2 * kWaves];
   __shared__ Coef sk;
@@ -558,6 +583,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) 
   for_channel_elements<EMAX>(g, [&](int k, size_t off) {
     v[k] = __builtin_nontemporal_load(xc + off);
     gq[k] = __builtin_nontemporal_load(dyc + off);
+    if constexpr (kRelu) gq[k] = mask1(gq[k], __builtin_nontemporal_load(a.ry + (size_t)c * g.HW + off));
   });
   double s_dy = 0.0, s_dyxmu = 0.0;
   for_channel_elements<EMAX>(g, [&](int k, size_t) {
@@ -648,8 +674,16 @@ int check_shape(const char* fn, int N, int C, int HW) {
 
 template <int kKind>
 void launch_reduce(int mode, dim3 grid, const float* x, const float* dy, const float* mean, double2* partial,
-                   const Geometry& g) {
+                   const Geometry& g, const float* ry = nullptr) {
   hipStream_t st = tt::stream();
+  if constexpr (kKind == 1) {
+    if (ry) {   // backward behind a fused ReLU: dy is masked by (ry > 0) as it is read
+      if (mode == 3) bn_reduce_stream<1, true><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g, ry);
+      if (mode == 1) bn_reduce_flat<1, 4, true><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g, ry);
+      if (mode == 2) bn_reduce_flat<1, 1, true><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g, ry);
+      return;
+    }
+  }
   if (mode == 0) bn_reduce_planes<kKind><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
   if (mode == 3) bn_reduce_stream<kKind><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
   if (mode == 1) bn_reduce_flat<kKind, 4><<<grid, kThreads, 0, st>>>(x, dy, mean, partial, g);
@@ -720,7 +754,7 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
                         float* save_mean, float* save_var_eps, float* save_sd, const float* running_mean_in,
                         const float* running_var_in, float* running_mean_out, float* running_var_out,
                         float* num_batches_tracked, double momentum, double eps, int N, int C, int HW,
-                        double2* fixed_partials, size_t fixed_capacity) {
+                        double2* fixed_partials, size_t fixed_capacity, bool relu = false) {
   TT_REQUIRE_INIT();
   if (check_shape(fn, N, C, HW)) return -1;
   TT_REQUIRE(x && y && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
@@ -746,8 +780,13 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
   if (const int cap = small_channel_capacity(N, C, HW)) {
     tt::ProfScope prof(timed ? TT_PROF_BN_FWD_APPLY : -1);
     const Geometry gs = small_geometry(N, C, HW);
-    if (cap == 16) bn_fwd_small<16><<<C, kThreads, 0, st>>>(a, gs);
-    else bn_fwd_small<kSmallMax><<<C, kThreads, 0, st>>>(a, gs);
+    if (relu) {
+      if (cap == 16) bn_fwd_small<16, true><<<C, kThreads, 0, st>>>(a, gs);
+      else bn_fwd_small<kSmallMax, true><<<C, kThreads, 0, st>>>(a, gs);
+    } else {
+      if (cap == 16) bn_fwd_small<16><<<C, kThreads, 0, st>>>(a, gs);
+      else bn_fwd_small<kSmallMax><<<C, kThreads, 0, st>>>(a, gs);
+    }
     TT_LAUNCH_CHECK();
     return 0;
   }
@@ -777,9 +816,15 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
   a.partial_splits = gr.splits;
   {
     tt::ProfScope prof(timed ? TT_PROF_BN_FWD_APPLY : -1);
-    if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
-    if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
-    if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+    if (relu) {
+      if (mode == 0) bn_fwd_apply<0, true><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 1) bn_fwd_apply<1, true><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 2) bn_fwd_apply<2, true><<<grid, kThreads, 0, st>>>(a, g);
+    } else {
+      if (mode == 0) bn_fwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 1) bn_fwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 2) bn_fwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+    }
   }
   TT_LAUNCH_CHECK();
   return 0;
@@ -792,6 +837,15 @@ int tt_bn_fwd_train_f32(const float* x, const float* gamma, const float* beta, f
   return bn_fwd_train("tt_bn_fwd_train_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd, running_mean_in,
                       running_var_in, running_mean_out, running_var_out, num_batches_tracked, momentum, eps, N, C, HW,
                       nullptr, 0);
+}
+
+int tt_bn_relu_fwd_train_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
+                             float* save_var_eps, float* save_sd, const float* running_mean_in,
+                             const float* running_var_in, float* running_mean_out, float* running_var_out,
+                             float* num_batches_tracked, double momentum, double eps, int N, int C, int HW) {
+  return bn_fwd_train("tt_bn_relu_fwd_train_f32", x, gamma, beta, y, save_mean, save_var_eps, save_sd, running_mean_in,
+                      running_var_in, running_mean_out, running_var_out, num_batches_tracked, momentum, eps, N, C, HW,
+                      nullptr, 0, true);
 }
 
 int tt_bn_fwd_train_noalloc_f32(const float* x, const float* gamma, const float* beta, float* y, float* save_mean,
@@ -836,20 +890,27 @@ int tt_bn_fwd_eval_f32(const float* x, const float* gamma, const float* beta, fl
   return 0;
 }
 
-int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
-                  const float* save_var_eps, const float* save_sd, float* dx, float* dgamma, float* dbeta, int N,
-                  int C, int HW) {
+// Backward behind tt_bn_bwd_f32 (ry == nullptr) and tt_bn_relu_bwd_f32 (ry = the fused ReLU's output).
+static int bn_bwd(const char* fn, const float* x, const float* dy, const float* ry, const float* gamma,
+                  const float* save_mean, const float* save_var_eps, const float* save_sd, float* dx, float* dgamma,
+                  float* dbeta, int N, int C, int HW) {
   TT_REQUIRE_INIT();
-  if (check_shape("tt_bn_bwd_f32", N, C, HW)) return -1;
-  TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "tt_bn_bwd_f32: null tensor pointer");
-  TT_REQUIRE_ALIGNED("tt_bn_bwd_f32", x, dy, dx);
+  if (check_shape(fn, N, C, HW)) return -1;
+  TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
+  TT_REQUIRE_ALIGNED(fn, x, dy, dx, ry);
   if (!dx && !dgamma && !dbeta) return 0;
   if (const int cap = small_channel_capacity(N, C, HW)) {
     tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
     const Geometry gs = small_geometry(N, C, HW);
-    BwdArgs b{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, nullptr, 0};
-    if (cap == 16) bn_bwd_small<16><<<C, kThreads, 0, tt::stream()>>>(b, gs);
-    else bn_bwd_small<kSmallMax><<<C, kThreads, 0, tt::stream()>>>(b, gs);
+    BwdArgs b{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, nullptr, 0, ry};
+    hipStream_t st = tt::stream();
+    if (ry) {
+      if (cap == 16) bn_bwd_small<16, true><<<C, kThreads, 0, st>>>(b, gs);
+      else bn_bwd_small<kSmallMax, true><<<C, kThreads, 0, st>>>(b, gs);
+    } else {
+      if (cap == 16) bn_bwd_small<16><<<C, kThreads, 0, st>>>(b, gs);
+      else bn_bwd_small<kSmallMax><<<C, kThreads, 0, st>>>(b, gs);
+    }
     TT_LAUNCH_CHECK();
     return 0;
   }
@@ -862,19 +923,39 @@ int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const flo
   dim3 grid(g.splits, C);
   {
     tt::ProfScope prof(TT_PROF_BN_BWD_REDUCE);
-    launch_reduce<1>(rmode, dim3(gr.splits, C), x, dy, save_mean, (double2*)ws, gr);
+    launch_reduce<1>(rmode, dim3(gr.splits, C), x, dy, save_mean, (double2*)ws, gr, ry);
   }
   TT_LAUNCH_CHECK();
-  BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws, gr.splits};
+  BwdArgs a{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, (const double2*)ws, gr.splits, ry};
   hipStream_t st = tt::stream();
   {
     tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
-    if (mode == 0) bn_bwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
-    if (mode == 1) bn_bwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
-    if (mode == 2) bn_bwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+    if (ry) {
+      if (mode == 0) bn_bwd_apply<0, true><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 1) bn_bwd_apply<1, true><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 2) bn_bwd_apply<2, true><<<grid, kThreads, 0, st>>>(a, g);
+    } else {
+      if (mode == 0) bn_bwd_apply<0><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 1) bn_bwd_apply<1><<<grid, kThreads, 0, st>>>(a, g);
+      if (mode == 2) bn_bwd_apply<2><<<grid, kThreads, 0, st>>>(a, g);
+    }
   }
   TT_LAUNCH_CHECK();
   return 0;
+}
+
+int tt_bn_bwd_f32(const float* x, const float* dy, const float* gamma, const float* save_mean,
+                  const float* save_var_eps, const float* save_sd, float* dx, float* dgamma, float* dbeta, int N,
+                  int C, int HW) {
+  return bn_bwd("tt_bn_bwd_f32", x, dy, nullptr, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, N, C, HW);
+}
+
+int tt_bn_relu_bwd_f32(const float* x, const float* dy, const float* relu_y, const float* gamma, const float* save_mean,
+                       const float* save_var_eps, const float* save_sd, float* dx, float* dgamma, float* dbeta, int N,
+                       int C, int HW) {
+  TT_REQUIRE(relu_y != nullptr, "tt_bn_relu_bwd_f32: null ReLU output");
+  return bn_bwd("tt_bn_relu_bwd_f32", x, dy, relu_y, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, N, C,
+                HW);
 }
 
 int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {

@@ -110,6 +110,90 @@ def bn_fwd_train(x, gamma, beta, running_mean, running_var, momentum, eps, num_b
     return y, mean, var_eps, sd, new_rm, new_rv
 
 
+class DeferredBatchNorm:
+    """A training forward that has not been launched yet (see ``_hip.defer``).  ``run()`` launches
+    it as it is; ``run_with_relu(out)`` launches the variant whose output is ``maximum(y, 0)`` --
+    into ``out``, or into the normalisation's own array when ``out`` is None (an in-place ReLU).
+    When the ReLU's result went elsewhere, the normalised values themselves were never stored:
+    their array recomputes them (same kernels, same bits, scratch statistics, no running update)
+    should anybody ask for it."""
+
+    def __init__(self, x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked):
+        self.x, self.gamma, self.beta = x, gamma, beta
+        self.momentum, self.eps = float(momentum if momentum is not None else 0.0), float(eps)
+        self.nbt = num_batches_tracked
+        self.dims = n, c, hw = _nchw(x)
+        self.y = hiparray.lazy(x.shape)
+        self.stats = [hiparray.empty((c,)) for _ in range(3)]        # mean, var + eps, sd
+        self.track = running_mean is not None and running_var is not None
+        self.rm_in, self.rv_in = (running_mean, running_var) if self.track else (None, None)
+        self.new_rm = hiparray.empty((c,)) if self.track else None
+        self.new_rv = hiparray.empty((c,)) if self.track else None
+
+    def _launch(self, entry, out):
+        mean, var_eps, sd = self.stats
+        _hip.call(entry, self.x.ptr, _ptr(self.gamma), _ptr(self.beta), out.ptr, mean.ptr, var_eps.ptr, sd.ptr,
+                  _ptr(self.rm_in), _ptr(self.rv_in), _ptr(self.new_rm), _ptr(self.new_rv), _ptr(self.nbt),
+                  self.momentum, self.eps, *self.dims)
+
+    def run(self):
+        self._launch('tt_bn_fwd_train_f32', self.y)
+
+    def run_with_relu(self, out=None):
+        if out is None:
+            self._launch('tt_bn_relu_fwd_train_f32', self.y)
+            return self.y
+        self._launch('tt_bn_relu_fwd_train_f32', out)
+        x, gamma, beta, eps, dims = self.x, self.gamma, self.beta, self.eps, self.dims
+
+        def recompute(buf):
+            scratch = [hiparray.empty((dims[1],)) for _ in range(3)]
+            _hip.call('tt_bn_fwd_train_f32', x.ptr, _ptr(gamma), _ptr(beta), buf.ptr, scratch[0].ptr, scratch[1].ptr,
+                      scratch[2].ptr, None, None, None, None, None, 0.0, eps, *dims)
+        self.y._buf.on_demand = recompute
+        return out
+
+
+def bn_fwd_train_deferred(x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None):
+    """``bn_fwd_train`` with the launch parked for the next operation to absorb (a ReLU) or to
+    trigger (anything else).  Same return value; the arrays are filled when the launch happens."""
+    _f32(x, gamma, beta, running_mean, running_var)
+    op = DeferredBatchNorm(x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked)
+    _hip.defer(op)
+    return (op.y, *op.stats, op.new_rm, op.new_rv)
+
+
+class DeferredReluBackward:
+    """``dy * (y > 0)`` not launched yet: a BatchNorm backward that comes next forms the product
+    itself while it reads ``dy`` (``bn_relu_bwd``); anything else finds it computed."""
+
+    def __init__(self, dy, y):
+        self.dy, self.y = dy, y
+        self.out = hiparray.lazy(y.shape)
+
+    def run(self):
+        _hip.call('tt_relu_bwd_f32', self.dy.ptr, self.y.ptr, self.out.ptr, self.y.size)
+
+
+def relu_bwd_deferred(dy, y):
+    _f32(dy, y)
+    op = DeferredReluBackward(dy, y)
+    _hip.defer(op)
+    return op.out
+
+
+def bn_relu_bwd(x, dy, relu_y, gamma, mean, var_eps, sd, need=(True, True, True)):
+    """``bn_bwd`` on the gradient ``dy * (relu_y > 0)``, masked as it is read."""
+    _f32(x, dy, relu_y, gamma)
+    n, c, hw = _nchw(x)
+    dx = hiparray.empty(x.shape) if need[0] else None
+    dgamma = hiparray.empty((c,)) if need[1] else None
+    dbeta = hiparray.empty((c,)) if need[2] else None
+    _hip.call('tt_bn_relu_bwd_f32', x.ptr, dy.ptr, relu_y.ptr, _ptr(gamma), mean.ptr, var_eps.ptr, sd.ptr,
+              _ptr(dx), _ptr(dgamma), _ptr(dbeta), n, c, hw)
+    return dx, dgamma, dbeta
+
+
 def bn_fwd_eval(x, gamma, beta, mean_in, var_in, eps):
     """Normalisation with given statistics (autograd/grad_nn.py:931-959)."""
     _f32(x, gamma, beta, mean_in, var_in)

@@ -56,20 +56,41 @@ class Device:
 
 class _Buffer:
     """One ``tt_malloc`` allocation; freed (returned to the library's pool) with the last array
-    that refers to it."""
-    __slots__ = ('ptr', 'nbytes')
+    that refers to it.  With ``lazy`` the block is taken on the first use of ``ptr``, and
+    ``on_demand`` (a callable receiving the buffer) then fills it: the output of an operation that
+    was absorbed into its successor exists only if somebody else asks for it."""
+    __slots__ = ('_ptr', 'nbytes', 'on_demand')
 
-    def __init__(self, nbytes):
-        p = ctypes.c_void_p()
-        _hip.call('tt_malloc', ctypes.byref(p), nbytes)
-        self.ptr = p.value or 0
+    def __init__(self, nbytes, lazy=False):
         self.nbytes = nbytes
+        self._ptr = 0
+        self.on_demand = None
+        if not lazy:
+            self._allocate()
+
+    def _allocate(self):
+        p = ctypes.c_void_p()
+        _hip.call('tt_malloc', ctypes.byref(p), self.nbytes)
+        self._ptr = p.value or 0
+
+    @property
+    def ptr(self):
+        if not self._ptr and self.nbytes:
+            # a parked operation may be the one that produces this very buffer: let it run (and
+            # allocate the buffer itself) before the block is taken here
+            _hip.flush()
+            if not self._ptr:
+                self._allocate()
+        if self.on_demand is not None:
+            fill, self.on_demand = self.on_demand, None
+            fill(self)
+        return self._ptr
 
     def __del__(self):
         try:
-            if self.ptr:
-                _hip.load_library().tt_free(ctypes.c_void_p(self.ptr))
-                self.ptr = 0
+            if self._ptr:
+                _hip.load_library().tt_free(ctypes.c_void_p(self._ptr))
+                self._ptr = 0
         except Exception:   # interpreter shutdown
             pass
 
@@ -103,6 +124,13 @@ class hiparray:
         shape = (shape,) if isinstance(shape, int) else tuple(shape)
         dtype = np.dtype(dtype)
         return cls(_buf=_Buffer(prod(shape) * dtype.itemsize), _shape=shape, dtype=dtype)
+
+    @classmethod
+    def lazy(cls, shape, dtype=np.float32):
+        """An array whose block is allocated when its ``ptr`` is first used."""
+        shape = (shape,) if isinstance(shape, int) else tuple(shape)
+        dtype = np.dtype(dtype)
+        return cls(_buf=_Buffer(prod(shape) * dtype.itemsize, lazy=True), _shape=shape, dtype=dtype)
 
     @classmethod
     def zeros(cls, shape, dtype=np.float32):
@@ -160,7 +188,7 @@ class hiparray:
         return self._shape[0]
 
     def __repr__(self):
-        return f'hiparray(shape={self._shape}, dtype={self._dtype}, ptr=0x{self.ptr:x})'
+        return f'hiparray(shape={self._shape}, dtype={self._dtype}, ptr=0x{self._buf._ptr:x})'
 
     # ---- data movement --------------------------------------------------------------------
     def get(self):
