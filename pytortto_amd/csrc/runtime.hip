@@ -269,7 +269,7 @@ int tt_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes) {
   if (bytes == 0) return 0;
   TT_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, S().stream));
   TT_HIP(hipStreamSynchronize(S().stream));
-  return 0;
+  return tt::conv_check_async_error();
 }
 
 int tt_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes) {
@@ -303,7 +303,7 @@ int tt_get_conv_math(int* mode) {
 int tt_sync(void) {
   TT_REQUIRE_INIT();
   TT_HIP(hipStreamSynchronize(S().stream));
-  return 0;
+  return tt::conv_check_async_error();
 }
 
 int tt_profile_enable(int on) {

@@ -42,6 +42,8 @@ int bn_scratch_init(int device);
 // tables of the weight gradient (conv_wgrad.hip); the caller has synchronised the stream.
 int conv_release_tables();
 int wgrad_release_tables();
+// After a stream sync: reports (once) a convolution launch whose blocks gave up waiting for each other.
+int conv_check_async_error();
 
 // Brackets the launches made during its lifetime with events when profiling is enabled
 // (a negative kernel id switches it off for that scope).
