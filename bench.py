@@ -48,9 +48,9 @@ BATCH = 64
 # x1.0).  Counters cannot be read from inside this script, so the figures of the last counter
 # run are carried here; the summary with the commands is in the profiles directory
 # (bench_hbm_traffic_fetch_write_size.txt).
-IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 209.6e6      # igemm_f32 + igemm_multi_f32 + igemm_fixup, mean over the 106 launches of a step (106.9e6 algorithmic)
-BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.3e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
-MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH = 314.6e6    # dy + taps read, dx written (308.3e6 algorithmic)
+IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 170.0e6      # igemm_f32 + igemm_multi_f32, mean over the 106 launches of a step (106.9e6 algorithmic)
+BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.2e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
+MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH = 311.7e6    # dy + taps read, dx written (308.3e6 algorithmic)
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
 
 
@@ -449,6 +449,8 @@ def main():
     ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
     ap.add_argument('--model-step-only', action='store_true',
                     help='run only the whole-network ResNet-50 training step and print its object (for profiling)')
+    ap.add_argument('--no-per-layer', action='store_true',
+                    help='skip the per-layer table (profiling runs: keeps the launch counts of a trace to whole steps)')
     ap.add_argument('--per-layer-only', action='store_true',
                     help='print only the per-layer table of the 23 ResNet-50 convolution shapes (for profiling)')
     ap.add_argument('--stack-only', choices=('preact', 'dcgan'),
@@ -517,7 +519,7 @@ def main():
     n_wg, ms_wg = prof['conv_wgrad']
     wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
     kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
-    layer_rows = per_layer_table(_hip, call, layers, 20)
+    layer_rows = None if args.no_per_layer else per_layer_table(_hip, call, layers, 20)
 
     # optional reduced-precision variant, reported separately and never part of `value`: the three
     # passes on bf16 MFMA (operands rounded inside the kernels, fp32 accumulation and tensors)
