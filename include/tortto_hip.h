@@ -339,6 +339,9 @@ int tt_leaky_relu_fwd_f32(const float* x, float* y, float negative_slope, size_t
 int tt_leaky_relu_bwd_f32(const float* dy, const float* x, float* dx, float negative_slope, size_t n);
 /* out = a + b (residual Add, autograd/grad_fcn.py:177-203). */
 int tt_add_f32(const float* a, const float* b, float* out, size_t n);
+/* out = maximum(a + b, 0): the residual Add (grad_fcn.py:177-203) with the ReLU behind it
+ * (autograd/grad_nn.py:56) in one pass; bit-identical to tt_add_f32 followed by tt_relu_fwd_f32. */
+int tt_add_relu_f32(const float* a, const float* b, float* out, size_t n);
 /* acc += alpha * v: gradient accumulation `fn.grad[ind] += grad` (tensor.py:596-599,
  * autograd/function.py:88-93). */
 int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n);

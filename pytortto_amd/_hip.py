@@ -73,6 +73,7 @@ PROTOTYPES = {
     'tt_adam_step_f32': [_P, _P, _P, _P, _P, c_size_t, _I, c_double, c_double, c_double, c_double, c_double, _I, _I],
     'tt_adam_step_multi_f32': [_I, _P, _P, _P, _P, _P, _P, _P, c_double, c_double, c_double, c_double, c_double, _I, _I],
     'tt_add_f32': [_P, _P, _P, c_size_t],
+    'tt_add_relu_f32': [_P, _P, _P, c_size_t],
     'tt_axpy_f32': [c_float, _P, _P, c_size_t],
     'tt_add_scalar_f32': [_P, c_float, c_size_t],
     'tt_fill_f32': [_P, c_float, c_size_t],

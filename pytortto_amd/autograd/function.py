@@ -64,7 +64,8 @@ class AccumulateGrad(BackwardFunction):
         var = self.variable
         if var.grad is None:
             g = self.grad[0]
-            var.grad = g if g.__class__ is xparray.hiparray else np.ascontiguousarray(g)
+            # a leaf keeps its gradient beyond this pass: it must not stay an alias of another holder's
+            var.grad = g.own() if g.__class__ is xparray.hiparray else np.ascontiguousarray(g)
         else:
             var.grad += self.grad[0]
 

@@ -69,7 +69,7 @@ class Add(Function):
         if a.__class__ is not hiparray:
             y = np.add(a, b)
         elif a.shape == b.shape:
-            y = ops.add(a, b)
+            y = ops.add_deferred(a, b)      # parked: a ReLU that comes next absorbs it
         elif b.size < a.size and _trailing(b.shape, a.shape):
             y = ops.add_rowvec(a, b)
         elif a.size < b.size and _trailing(a.shape, b.shape):
@@ -88,13 +88,15 @@ class Add(Function):
             # Every operand receives an array of its own, as the reference's reverse_broadcast does
             # (its ``sum((), keepdims=True)`` copies): gradients are stored by reference further on
             # and some backward functions scale theirs in place (LeakyRelu, grad_nn.py:92-94), so a
-            # shared array would hand one branch the other's already-masked gradient.
+            # shared array would hand one branch the other's already-masked gradient.  The second
+            # array is an alias that turns into a copy only if its holder writes it in place
+            # (``hiparray.own``): a residual branch that only reads its gradient copies nothing.
             need_a, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
 
             def back(shape, fresh):
                 if shape != g.shape:
                     return ops.sum_rows(g, prod(shape)).reshape(shape)
-                return g.copy() if fresh else g
+                return g.alias() if fresh else g
             ga = back(sa, False) if need_a else None
             gb = back(sb, need_a and sa == g.shape) if need_b else None
             return ga, gb

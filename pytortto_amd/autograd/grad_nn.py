@@ -195,6 +195,14 @@ class Relu(Function):
             else:
                 yt0 = build_links(_hip.take_pending().run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
             ctx.params['after_batch_norm'] = True
+        elif parked.__class__ is ops.DeferredAdd and parked.out._buf is xd0._buf:
+            # the input is a residual sum that has not been launched yet: maximum(a + b, 0) in one pass
+            if inplace:
+                inplace_precheck(xt0)
+                _hip.take_pending().run_with_relu()
+                yt0 = inplace_update(xt0, ctx)
+            else:
+                yt0 = build_links(_hip.take_pending().run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
         elif xd0.__class__ is hiparray:
             if inplace:
                 inplace_precheck(xt0)

@@ -6,7 +6,7 @@ namespace {
 
 constexpr int kThreads = 256;
 
-enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill, kLeakyRelu, kLeakyReluBwd, kAddScalar };
+enum Op { kRelu, kReluBwd, kAdd, kAxpy, kFill, kLeakyRelu, kLeakyReluBwd, kAddScalar, kAddRelu };
 
 template <int OP>
 __device__ __forceinline__ float apply1(float a, float b, float alpha) {
@@ -21,6 +21,10 @@ __device__ __forceinline__ float apply1(float a, float b, float alpha) {
   // non-finite gradient at a masked element gives NaN and a negative one -0, not +0
   if (OP == kReluBwd) return a * (b > 0.f ? 1.f : 0.f);
   if (OP == kAdd) return a + b;
+  if (OP == kAddRelu) {                           // maximum(a + b, 0): the sum rounded as by kAdd, NaN kept as by kRelu
+    const float t = a + b;
+    return (t > 0.f || t != t) ? t : 0.f;
+  }
   if (OP == kAxpy) return fmaf(alpha, a, b);      // a = v, b = acc
   if (OP == kAddScalar) return a + alpha;
   return alpha;                                    // kFill
@@ -31,8 +35,8 @@ __global__ __launch_bounds__(kThreads) void eltwise(const float* __restrict__ a,
                                                     float* __restrict__ out, float alpha, size_t n) {
   constexpr bool kUseA = OP != kFill;
   // results that are not accumulated in place stream out past the caches
-  constexpr bool kStreamOut = OP == kRelu || OP == kReluBwd || OP == kAdd || OP == kLeakyRelu || OP == kLeakyReluBwd;
-  constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy || OP == kLeakyReluBwd;
+  constexpr bool kStreamOut = OP == kRelu || OP == kReluBwd || OP == kAdd || OP == kLeakyRelu || OP == kLeakyReluBwd || OP == kAddRelu;
+  constexpr bool kUseB = OP == kReluBwd || OP == kAdd || OP == kAxpy || OP == kLeakyReluBwd || OP == kAddRelu;
   // two-input kernels whose inputs are read for the last time here (a gradient and the saved
   // activation, the two branches of a residual add) stream them in past the caches too: 8-9 %
   // faster than allocating loads at 200 MB per tensor; one-input kernels are faster with plain loads
@@ -97,6 +101,9 @@ int tt_leaky_relu_bwd_f32(const float* dy, const float* x, float* dx, float nega
   return run<kLeakyReluBwd>("tt_leaky_relu_bwd_f32", dy, x, dx, negative_slope, n);
 }
 int tt_add_f32(const float* a, const float* b, float* out, size_t n) { return run<kAdd>("tt_add_f32", a, b, out, 0.f, n); }
+int tt_add_relu_f32(const float* a, const float* b, float* out, size_t n) {
+  return run<kAddRelu>("tt_add_relu_f32", a, b, out, 0.f, n);
+}
 int tt_axpy_f32(float alpha, const float* v, float* acc, size_t n) {
   return run<kAxpy>("tt_axpy_f32", v, acc, acc, alpha, n);
 }

@@ -221,7 +221,7 @@ def bn_bwd(x, dy, gamma, mean, var_eps, sd, need=(True, True, True)):
 
 def relu_fwd(x, out=None):
     _f32(x)
-    y = hiparray.empty(x.shape) if out is None else out
+    y = hiparray.empty(x.shape) if out is None else out.own()
     _hip.call('tt_relu_fwd_f32', x.ptr, y.ptr, x.size)
     return y
 
@@ -235,14 +235,14 @@ def relu_bwd(dy, y):
 
 def leaky_relu_fwd(x, negative_slope, out=None):
     _f32(x)
-    y = hiparray.empty(x.shape) if out is None else out
+    y = hiparray.empty(x.shape) if out is None else out.own()
     _hip.call('tt_leaky_relu_fwd_f32', x.ptr, y.ptr, float(negative_slope), x.size)
     return y
 
 
 def leaky_relu_bwd(dy, x, negative_slope, out=None):
     _f32(dy, x)
-    dx = hiparray.empty(x.shape) if out is None else out
+    dx = hiparray.empty(x.shape) if out is None else out.own()
     _hip.call('tt_leaky_relu_bwd_f32', dy.ptr, x.ptr, dx.ptr, float(negative_slope), x.size)
     return dx
 
@@ -254,6 +254,37 @@ def add(a, b):
     out = hiparray.empty(a.shape)
     _hip.call('tt_add_f32', a.ptr, b.ptr, out.ptr, a.size)
     return out
+
+
+class DeferredAdd:
+    """``a + b`` of equal shapes, not launched yet (see ``_hip.defer``): a ReLU that comes next
+    computes ``maximum(a + b, 0)`` in one pass (``run_with_relu``); anything else finds the sum done.
+    When the ReLU's result went to an array of its own, the sum itself is produced on demand."""
+
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+        self.out = hiparray.lazy(a.shape)
+
+    def run(self):
+        _hip.call('tt_add_f32', self.a.ptr, self.b.ptr, self.out.ptr, self.a.size)
+
+    def run_with_relu(self, out=None):
+        a, b = self.a, self.b
+        if out is None:
+            _hip.call('tt_add_relu_f32', a.ptr, b.ptr, self.out.ptr, a.size)
+            return self.out
+        _hip.call('tt_add_relu_f32', a.ptr, b.ptr, out.ptr, a.size)
+        self.out._buf.on_demand = lambda buf: _hip.call('tt_add_f32', a.ptr, b.ptr, buf.ptr, a.size)
+        return out
+
+
+def add_deferred(a, b):
+    _f32(a, b)
+    if a.shape != b.shape:
+        raise ValueError(f'device add needs equal shapes, got {a.shape} and {b.shape}')
+    op = DeferredAdd(a, b)
+    _hip.defer(op)
+    return op.out
 
 
 # ---- MaxPool2d -------------------------------------------------------------------------------------

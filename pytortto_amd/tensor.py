@@ -219,6 +219,11 @@ class Tensor:
                         continue
                     if fn.grad[idx] is None:
                         fn.grad[idx] = g if g.__class__ is hiparray else np.ascontiguousarray(g)
+                    elif fn.grad[idx].__class__ is hiparray and fn.grad[idx]._shared and g.__class__ is hiparray:
+                        # the first arrival is an alias of somebody else's gradient (hiparray.alias):
+                        # the sum goes to a new array instead of copying it and adding in place
+                        from . import ops
+                        fn.grad[idx] = ops.add(fn.grad[idx], g)
                     else:
                         fn.grad[idx] += g
                 node.clear()

@@ -96,7 +96,7 @@ class _Buffer:
 
 
 class hiparray:
-    __slots__ = ('_buf', '_shape', '_dtype', '_version', '__weakref__')
+    __slots__ = ('_buf', '_shape', '_dtype', '_version', '_shared', '__weakref__')
 
     def __new__(cls, input_array=None, dtype=None, copy=True, _buf=None, _shape=None, _version=None):
         if input_array.__class__ is cls:
@@ -104,6 +104,7 @@ class hiparray:
                 return input_array
             input_array = input_array.get()
         self = object.__new__(cls)
+        self._shared = False
         if _buf is not None:            # internal: wrap an existing buffer
             self._buf, self._shape, self._dtype = _buf, tuple(_shape), np.dtype(dtype)
             self._version = _version if _version is not None else [0]
@@ -201,6 +202,27 @@ class hiparray:
     def item(self):
         return self.get().item()
 
+    def alias(self):
+        """A second array on the same block for a holder that only reads it.  Both arrays are marked
+        shared: whoever is about to write one of them in place (``+=``, ``fill``, ``set``, a kernel
+        with ``out=``) calls ``own()`` first, which moves that array to a copy.  Gradients handed to
+        two operands travel this way: each holder has an array of its own, as the reference's
+        copies give it, and the copy is made only for a holder that writes."""
+        self._shared = True
+        other = hiparray(_buf=self._buf, _shape=self._shape, dtype=self._dtype)
+        other._shared = True
+        return other
+
+    def own(self):
+        """Make sure this array is the only one on its block before it is written in place."""
+        if self._shared:
+            fresh = _Buffer(self.nbytes)
+            if self.nbytes:
+                _hip.call('tt_memcpy_d2d', fresh.ptr, self._buf.ptr, self.nbytes)
+            self._buf = fresh
+            self._shared = False
+        return self
+
     def copy(self):
         out = hiparray.empty(self._shape, self._dtype)
         if out.nbytes:
@@ -213,6 +235,7 @@ class hiparray:
         if host.shape != self._shape:
             host = np.broadcast_to(host, self._shape)
         host = np.ascontiguousarray(host)               # (a 0-d array comes back 1-d: same bytes)
+        self.own()
         if host.nbytes:
             _hip.call('tt_memcpy_h2d', self.ptr, host.ctypes.data, host.nbytes)
         return self
@@ -228,7 +251,9 @@ class hiparray:
             shape[i] = self.size // rest if rest else 0
         if prod(shape) != self.size:
             raise ValueError(f'cannot reshape array of size {self.size} into shape {tuple(shape)}')
-        return hiparray(_buf=self._buf, _shape=shape, dtype=self._dtype, _version=self._version)
+        view = hiparray(_buf=self._buf, _shape=shape, dtype=self._dtype, _version=self._version)
+        view._shared = self._shared
+        return view
 
     def view(self, _cls=None):
         return self
@@ -240,11 +265,13 @@ class hiparray:
 
     def fill(self, value):
         self._require_f32('fill')
+        self.own()
         if self.size:
             _hip.call('tt_fill_f32', self.ptr, float(value), self.size)
 
     def __iadd__(self, other):
         self._require_f32('+=')
+        self.own()
         if isinstance(other, hiparray):
             if other.shape != self._shape or other.dtype != self._dtype:
                 raise ValueError(f'device += needs equal shapes and dtypes, got {self._shape} and {other.shape}')

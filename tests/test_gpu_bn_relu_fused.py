@@ -181,3 +181,58 @@ def test_anything_but_a_relu_finds_the_parked_batchnorm_done():
     bn.eval()
     bn(tt.tensor(x).cuda())
     assert _hip.pending() is None
+
+
+@pytest.mark.parametrize('n', [1, 3, 4, 1023, 4099, (1 << 20) + 3])
+def test_add_relu_entry_point_matches_add_then_relu_bit_for_bit(n):
+    from pytortto_amd import _hip
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(n)
+    a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    if n >= 4:
+        a[:4] = [np.nan, np.inf, -np.inf, -0.0]
+        b[:4] = [1.0, -np.inf, 1.0, 0.0]
+    ad, bd, s, want, got = hiparray(a), hiparray(b), hiparray.empty((n,)), hiparray.empty((n,)), hiparray.empty((n,))
+    _hip.call('tt_add_f32', ad.ptr, bd.ptr, s.ptr, n)
+    _hip.call('tt_relu_fwd_f32', s.ptr, want.ptr, n)
+    _hip.call('tt_add_relu_f32', ad.ptr, bd.ptr, got.ptr, n)
+    _bits_equal(got.get(), want.get(), 'add_relu')
+    with np.errstate(invalid='ignore'):
+        _bits_equal(got.get(), np.maximum(a + b, 0), 'add_relu vs NumPy')
+
+
+@pytest.mark.parametrize('inplace', [False, True])
+def test_relu_after_a_residual_add_through_the_autograd_nodes(inplace):
+    """relu(a + b): the Add is parked and the ReLU absorbs it; the graph keeps AddBackward and
+    ReluBackward, both operands receive dy * (y > 0) in arrays of their own."""
+    import pytortto_amd as tt
+    from pytortto_amd import _hip, nn, ops
+    rng = np.random.default_rng(6)
+    a, b = rng.standard_normal((3, 4, 5, 7)).astype(np.float32), rng.standard_normal((3, 4, 5, 7)).astype(np.float32)
+    g = rng.standard_normal(a.shape).astype(np.float32)
+    at, bt = _leaf(a), _leaf(b)
+    s = at + bt
+    assert _hip.pending().__class__ is ops.DeferredAdd
+    out = nn.functional.relu(s, inplace=inplace)
+    assert _hip.pending() is None
+    assert out.grad_fn.__class__.__name__ == 'ReluBackward'
+    assert out.grad_fn.next_functions[0][0].__class__.__name__ == 'AddBackward'
+    out.backward(tt.tensor(g).cuda())
+    want = np.maximum(a + b, 0)
+    np.testing.assert_array_equal(out.cpu().detach().numpy(), want)
+    np.testing.assert_array_equal(at.grad.get(), g * (want > 0))
+    np.testing.assert_array_equal(bt.grad.get(), g * (want > 0))
+    assert at.grad.ptr != bt.grad.ptr
+    # a second consumer of the sum finds it computed on demand; anything but a ReLU finds it done
+    at, bt = _leaf(a), _leaf(b)
+    s = at + bt
+    out = nn.functional.relu(s) + s
+    np.testing.assert_array_equal(out.cpu().detach().numpy(), want + (a + b))
+    s2 = at + bt
+    np.testing.assert_array_equal(s2.data.get(), a + b)
+
+
+def _leaf(values):
+    import pytortto_amd as tt
+    from pytortto_amd.xparray import hiparray
+    return tt.Tensor(hiparray(np.ascontiguousarray(values, dtype=np.float32)), requires_grad=True)
