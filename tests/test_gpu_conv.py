@@ -234,3 +234,31 @@ def test_conv_is_bit_reproducible(case):
                    hiparray(rng.standard_normal((8, 8, 3, 3), dtype=np.float32)), None, (1, 1), (1, 1), (1, 1), 1)
     for a, b in zip(first, once()):
         np.testing.assert_array_equal(a, b)
+
+
+def test_stream_k_partial_sums_across_many_launches():
+    """The partial sums of a split tile pass from block to block through memory, announced by a flag
+    per block whose value changes from launch to launch.  Launches of different layers back to
+    back -- each re-using the same partial slots and flag words -- must give the same bits every
+    time, and the right ones: a partial read too early, or left over from the launch before, would
+    show here."""
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    geo = ((1, 1), (1, 1), (1, 1), 1)
+    rng = np.random.default_rng(21)
+    layers = []
+    for n, c, h, k in ((8, 128, 28, 128), (8, 256, 14, 256), (4, 512, 7, 512), (16, 64, 56, 64)):   # tiles: 49, 98 x ..., all split
+        x = rng.standard_normal((n, c, h, h), dtype=np.float32)
+        w = (rng.standard_normal((k, c, 3, 3)) / np.sqrt(9 * c)).astype(np.float32)
+        y_ref, _ = oracle.convolution_forward(x, w, None, *geo)
+        layers.append((hiparray(x), hiparray(w), y_ref))
+    outs = [[] for _ in layers]
+    for _ in range(12):
+        for i, (x, w, _) in enumerate(layers):
+            outs[i].append(ops.conv2d_fwd(x, w, None, *geo))        # enqueued back to back, read afterwards
+    _hip.synchronize()
+    for (x, w, y_ref), ys in zip(layers, outs):
+        first = ys[0].get()
+        np.testing.assert_allclose(first, y_ref, rtol=1e-4, atol=1e-5)
+        for y in ys[1:]:
+            np.testing.assert_array_equal(y.get(), first)
