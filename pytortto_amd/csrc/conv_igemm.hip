@@ -33,6 +33,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <type_traits>
 #include <vector>
 
 #include "tt_common.h"
@@ -50,7 +51,7 @@ constexpr int kInvalid = -(1 << 20);
 // One entry per reduction index k (padded with never-valid entries to a whole chunk).
 struct KEntry {
   int off;   // element offset added to the pixel's base offset (tap-mask tables: byte offset, biased to be >= 0)
-  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit (tap-mask tables: tap number, 31 = padding)
+  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit (tap-mask tables: tap number; 31, or 63 with the 64-bit mask, = padding)
 };
 
 typedef int intx2 __attribute__((ext_vector_type(2)));
@@ -81,6 +82,8 @@ struct Igemm {
   //                 itself; 16-byte buffer loads along pixels, kStride elements between k rows
   //   kModeTapMask: buffer loads; per tile every lane keeps one bit per tap (TB x TC <= 31 taps)
   //                 telling whether that tap falls outside the image for its pixel
+  //   kModeTapMask64: the same with a 64-bit mask (32 .. 63 taps: 7x7 kernels), one 64-bit shift
+  //                 per element instead of a 32-bit one
   // The two buffer modes address relative to the first image of the tile with 32-bit byte
   // offsets; the host selects them only when those stay below 2 GiB.
   int mode;
@@ -117,7 +120,7 @@ struct Igemm {
 // and they never share memory with per-call scratch data.
 struct KTabArgs {
   int Kred, Kpad, TB, TC, sa, sb, sc, stepH, stepW;
-  int tapMask;   // 1: entries are {4*(off + offBias), tap number b*TC + c}
+  int tapMask;   // 1 / 2: entries are {4*(off + offBias), tap number b*TC + c}; padding tap 31 / 63
   int offBias;
 };
 KEntry ktab_entry(const KTabArgs& a, int k) {
@@ -133,7 +136,7 @@ KEntry ktab_entry(const KTabArgs& a, int k) {
     }
   } else {
     e.off = 0;
-    e.dhw = a.tapMask ? 31 : (-16384) & 0xffff;   // tap 31 / a row far above the image: never valid
+    e.dhw = a.tapMask == 2 ? 63 : a.tapMask ? 31 : (-16384) & 0xffff;   // the mask's top tap / a row far above the image: never valid
   }
   return e;
 }
@@ -228,7 +231,7 @@ __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restr
 using tt::xcd_remap;
 
 typedef float floatx2 __attribute__((ext_vector_type(2)));
-constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2;
+constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2, kModeTapMask64 = 3;
 constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format
 constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out of range and read 0
 
@@ -269,6 +272,8 @@ template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT, bool BF>
 __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
+  constexpr bool MASK = MODE == kModeTapMask || MODE == kModeTapMask64;
+  using TapBits = std::conditional_t<MODE == kModeTapMask64, uint64_t, uint32_t>;
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ITEMS = (kBKQ * BM + kThreads - 1) / kThreads, B_ITEMS = kBKQ * BN / kThreads;
   static_assert(B_ITEMS >= 1 && kThreads % BM == 0 && kThreads % BN == 0, "tile shape");
@@ -296,7 +301,7 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   __amdgpu_buffer_rsrc_t srcSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.src, 0, kSrdRecords, kSrdFlags);
   const __amdgpu_buffer_rsrc_t wSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.wbuf, 0, kSrdRecords, kSrdFlags);
   int bvoff = 0, avoff = 0, asoff = 0;
-  uint32_t nmask = 0xffffffffu;   // bit t set: tap t lies outside the image for this lane's pixel
+  TapBits nmask = ~(TapBits)0;   // bit t set: tap t lies outside the image for this lane's pixel
   constexpr int AQ = kThreads / BM;   // k-quads between a thread's weight items
   auto set_tile = [&](int tile) __attribute__((always_inline)) {
     i0 = (tile % p.tilesI) * BM;
@@ -313,7 +318,7 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
       } else {
         const int m = m0 + pix;
         bvoff = 0;
-        nmask = 0xffffffffu;
+        nmask = ~(TapBits)0;
         if (m < p.M) {
           const uint32_t n = tt::fd_div((uint32_t)m, p.divUV);
           const uint32_t rem = (uint32_t)m - n * p.divUV.d;
@@ -321,11 +326,11 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
           const uint32_t v = rem - u * p.divV.d;
           const int ih = (int)u * p.su + p.bh, iw = (int)v * p.sv + p.bw;
           bvoff = 4 * ((int)(n - n0) * p.srcStrideN + ih * p.srcRow + iw + p.voffBias);
-          uint32_t cols = 0, inside = 0;
-          for (int c = 0; c < p.TC; ++c) cols |= (uint32_t)((unsigned)(iw + c * p.stepW) < (unsigned)p.Wlim) << c;
+          TapBits cols = 0, inside = 0;
+          for (int c = 0; c < p.TC; ++c) cols |= (TapBits)((unsigned)(iw + c * p.stepW) < (unsigned)p.Wlim) << c;
           for (int b = 0; b < p.TB; ++b)
             if ((unsigned)(ih + b * p.stepH) < (unsigned)p.Hlim) inside |= cols << (b * p.TC);
-          nmask = ~inside;   // bit 31 (the padding entries' tap) always stays set: TB*TC <= 31
+          nmask = ~inside;   // the top bit (the padding entries' tap) always stays set: TB*TC <= 31 or 63
         }
       }
       if constexpr (AT) {   // w[k][c] in place: k = Kred rows of I = C/groups columns per group
@@ -413,9 +418,9 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   };
   auto load_b_elem = [&](int e) __attribute__((always_inline)) {   // uses tab_e: must follow load_tab() of the same chunk
     const intx2 t = tab_e[e];
-    if constexpr (MODE == kModeTapMask) {
+    if constexpr (MASK) {
       // {byte offset, tap}: shift the lane's "outside" bit for this tap into bit 31 of its offset
-      const uint32_t vo = ((nmask >> t.y) << 31) | (uint32_t)bvoff;
+      const uint32_t vo = ((uint32_t)(nmask >> t.y) << 31) | (uint32_t)bvoff;
       breg[e >> 2][e & 3] = as_float(__builtin_amdgcn_raw_buffer_load_b32(srcSrd, (int)vo, t.x, 0));
       return;
     }
@@ -968,13 +973,17 @@ void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   else if (p.mode == kModeGemm) launch_mode<WM, WN, MT, NT, kModeGemm, false>(p, groups, sk_blocks, st);
   else if (p.mode == kModeTapMask && at) launch_mode<WM, WN, MT, NT, kModeTapMask, true>(p, groups, sk_blocks, st);
   else if (p.mode == kModeTapMask) launch_mode<WM, WN, MT, NT, kModeTapMask, false>(p, groups, sk_blocks, st);
+  else if (p.mode == kModeTapMask64) launch_mode<WM, WN, MT, NT, kModeTapMask64, false>(p, groups, sk_blocks, st);
   else launch_mode<WM, WN, MT, NT, kModeCompare, false>(p, groups, sk_blocks, st);
 }
 
 // Picks how the kernel addresses the gathered operand (see Igemm::mode) and completes the table
 // arguments accordingly.  Needs the source geometry fields of `p`; `pixels` = U*V pixels per
 // image, `gemm_geometry` = 1x1 / stride 1 / unpadded / pixel count a multiple of 4.
-void choose_mode(Igemm& p, KTabArgs& ka, bool gemm_geometry, int N, int U, int V, long long weight_bytes) {
+// `wide_masks`: the launch may use the 64-bit tap mask (single launches only: the shared grids of
+// an input gradient's stride-parity classes are built for the other modes).
+void choose_mode(Igemm& p, KTabArgs& ka, bool gemm_geometry, int N, int U, int V, long long weight_bytes,
+                 bool wide_masks = false) {
   p.mode = kModeCompare;
   p.TB = ka.TB; p.TC = ka.TC; p.stepH = ka.stepH; p.stepW = ka.stepW;
   const long long b1 = (long long)(p.bh < 0 ? -p.bh : 0) * p.srcRow + (p.bw < 0 ? -p.bw : 0);
@@ -990,11 +999,11 @@ void choose_mode(Igemm& p, KTabArgs& ka, bool gemm_geometry, int N, int U, int V
   if (reach >= limit || weight_bytes >= limit) return;
   if (gemm_geometry && ka.Kred % (4 * kBKQ) == 0) {
     p.mode = kModeGemm;
-  } else if (ka.TB * ka.TC <= 31) {
-    p.mode = kModeTapMask;
+  } else if (ka.TB * ka.TC <= 31 || (wide_masks && ka.TB * ka.TC <= 63)) {
+    p.mode = ka.TB * ka.TC <= 31 ? kModeTapMask : kModeTapMask64;
     p.voffBias = (int)b1;
     p.srdBias = b1 + b2;
-    ka.tapMask = 1;
+    ka.tapMask = ka.TB * ka.TC <= 31 ? 1 : 2;
     ka.offBias = (int)b2;
   }
 }
@@ -1140,13 +1149,15 @@ int cached_table(const std::vector<int>& key, const void* host, size_t bytes, co
 int check_ktab(const char* fn, const Igemm& p, const KTabArgs& ka, const std::vector<KEntry>& tab, int N, int groups,
                int U, int V, int planes, long long src_elems) {
   if (p.mode == kModeGemm) return 0;   // plain matrix product: no table is read
-  const bool mask = p.mode == kModeTapMask;
+  const bool mask = p.mode == kModeTapMask || p.mode == kModeTapMask64;
+  const int top_tap = p.mode == kModeTapMask64 ? 63 : 31;
   TT_REQUIRE((int)tab.size() == ka.Kpad && ka.Kpad % (4 * kBKQ) == 0 && ka.Kred <= ka.Kpad,
              "%s: index table of %zu entries for a reduction of %d (%d padded)", fn, tab.size(), ka.Kred, ka.Kpad);
   TT_REQUIRE(p.srcRow == p.Wlim && (long long)p.srcStrideG == (long long)planes * p.Hlim * p.Wlim &&
                  (long long)N * p.srcStrideN <= src_elems,
              "%s: source geometry of the launch does not describe an [N, C, %d, %d] tensor", fn, p.Hlim, p.Wlim);
-  TT_REQUIRE(!mask || ka.TB * ka.TC <= 31, "%s: %d x %d taps do not fit the 31-bit tap mask", fn, ka.TB, ka.TC);
+  TT_REQUIRE(!mask || (ka.TB * ka.TC <= top_tap && ka.tapMask == (top_tap == 63 ? 2 : 1)),
+             "%s: %d x %d taps do not fit the %d-bit tap mask", fn, ka.TB, ka.TC, top_tap);
   const long long plane = (long long)p.Hlim * p.Wlim;
   // images a 256-pixel tile can span beyond its first one (buffer offsets are relative to that)
   const long long span = std::min<long long>(N - 1, 255 / ((long long)U * V) + 1);
@@ -1157,7 +1168,7 @@ int check_ktab(const char* fn, const Igemm& p, const KTabArgs& ka, const std::ve
     if (mask) {
       const int tap = e.dhw;
       if (k >= ka.Kred) {
-        TT_REQUIRE(tap == 31, "%s: padding entry %d of the index table names tap %d", fn, k, tap);
+        TT_REQUIRE(tap == top_tap, "%s: padding entry %d of the index table names tap %d", fn, k, tap);
         continue;
       }
       TT_REQUIRE(tap >= 0 && tap < ka.TB * ka.TC && e.off >= 0 && e.off % 4 == 0,
@@ -1380,7 +1391,7 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
   p.Kred = Kred;
   KTabArgs ka{Kred, KQ * 4, R, S, H * W, dh * W, dw, dh, dw, 0, 0};
   choose_mode(p, ka, plain && (H * W) % 4 == 0, N, P, Q,
-              in_place ? (long long)sizeof(float) * K * Kred : (long long)wp_bytes);
+              in_place ? (long long)sizeof(float) * K * Kred : (long long)wp_bytes, true);
   if (make_ktab(fn, p, ka, N, groups, P, Q, Cg, (long long)N * C * H * W, check_only, &p.ktab)) return -1;
   if (check_only) return 0;
   if (!in_place) {
@@ -1499,7 +1510,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       p.ou = cellH; p.ouh = 0; p.ov = cellW; p.ovw = 0;
       p.outH = Hx; p.outW = Wx;
       KTabArgs ka{Kred, KQ * 4, Na, Nb, P * Q, Q, 1, 1, 1, 0, 0};
-      choose_mode(p, ka, false, N, U, V, (long long)wp_bytes);
+      choose_mode(p, ka, false, N, U, V, (long long)wp_bytes, true);
       // (one group: the launch's group stride is 0, the check takes the whole of dy as one group)
       Igemm pc = p;
       pc.srcStrideG = K * P * Q;

@@ -18,10 +18,12 @@
 // each load adds a per-lane constant (row / column offset), padding taps set bit 31 of the
 // offset from a per-chunk tap mask and read 0 through the buffer range check, and nothing is
 // masked when the values are written to LDS.  Offsets are relative to the first image of the
-// chunk; geometries whose offsets could reach 2 GiB, or with more than 31 taps, take the
+// chunk.  Kernels of 32 to 63 taps (7x7) keep a 64-bit mask (WIDE: its upper half comes from a second
+// table); geometries whose offsets could reach 2 GiB, or with more than 63 taps, take the
 // compare-and-select path instead.
 #include <algorithm>
 #include <map>
+#include <type_traits>
 #include <vector>
 
 #include "tt_common.h"
@@ -58,6 +60,7 @@ struct Wgrad {
   // buffer path: per output pixel m {image n, 4*(p*Q + q), 4*(ih*W + iw + xBias), tap mask};
   // entries from M to chunks*32 hold {N-1, bit 31, 0, all ones}.  Built once per geometry.
   const int4* pixtab;
+  const int* pixhi;   // kernels of 32 .. 63 taps: bits 32 .. 63 of every pixel's tap mask
 };
 
 constexpr int kSrdFlags = 0x00020000;     // raw buffer, 32-bit data format
@@ -75,12 +78,42 @@ __device__ __forceinline__ uint32_t tap_range_bits(int pos, int lim, int n, int 
   return lo > hi ? 0u : upto & ~below;
 }
 
+// The same for masks of up to 63 bits (n*unit <= 63).
+__device__ __forceinline__ uint64_t tap_range_bits64(int pos, int lim, int n, int unit, const tt::FastDiv& step) {
+  int lo = pos >= 0 ? 0 : (int)tt::fd_div((uint32_t)(-pos + (int)step.d - 1), step);
+  const int room = lim - 1 - pos;
+  const int hi = room < 0 ? -1 : min(n - 1, (int)tt::fd_div((uint32_t)room, step));
+  lo = min(lo, n);
+  const uint64_t upto = (1ull << ((hi + 1) * unit)) - 1ull, below = (1ull << (lo * unit)) - 1ull;
+  return lo > hi ? 0ull : upto & ~below;
+}
+
 // Pixel table of the buffer path: what the main loop would otherwise recompute for every chunk
 // in every block (two divisions, the tap ranges) depends only on the geometry.
-__global__ void wgrad_build_pixtab(int4* __restrict__ tab, Wgrad p, int entries, int N) {
+// `hi` (kernels of 32 .. 63 taps only): receives the upper half of each 64-bit mask.
+__global__ void wgrad_build_pixtab(int4* __restrict__ tab, int* __restrict__ hi, Wgrad p, int entries, int N) {
   const int m = blockIdx.x * blockDim.x + threadIdx.x;
   if (m >= entries) return;
   int4 e = make_int4(N - 1, (int)0x80000000u, 0, -1);
+  if (hi != nullptr) {
+    uint64_t outside = ~0ull;
+    if (m < p.M) {
+      const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
+      const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
+      const uint32_t pp = tt::fd_div(pq, p.divQ);
+      const uint32_t qq = pq - pp * p.divQ.d;
+      const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
+      uint64_t row_ones = 0;
+      for (int r = 0; r < p.R; ++r) row_ones |= 1ull << (r * p.S);
+      const uint64_t cols = tap_range_bits64(iw, p.W, p.S, 1, p.divDw);
+      const uint64_t rows = tap_range_bits64(ih, p.H, p.R, p.S, p.divDh) & row_ones;
+      outside = ~(cols * rows);   // bit 63 stays set: R*S <= 63
+      e = make_int4((int)n, 4 * (int)pq, 4 * (ih * p.W + iw + p.xBias), (int)(uint32_t)outside);
+    }
+    tab[m] = e;
+    hi[m] = (int)(uint32_t)(outside >> 32);
+    return;
+  }
   if (m < p.M) {
     const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
     const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
@@ -103,10 +136,12 @@ __global__ void wgrad_build_pixtab(int4* __restrict__ tab, Wgrad p, int entries,
 // unpadded layer, where x is indexed by the output pixel like dy and has no padding to mask.
 // BF: the optional bf16 variant (tt_set_conv_math): operands rounded to bfloat16 after the LDS
 // read, v_mfma_f32_32x32x16_bf16, float32 accumulation.
-template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB, bool BF>
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB, bool BF, bool WIDE = false>
 __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   static_assert(WM * WN == 4, "four waves per block");
   static_assert(BUF || (!VA && !VB), "vector fetches belong to the buffer path");
+  static_assert(!WIDE || (BUF && !VB), "64-bit tap masks belong to the buffer path of kernels larger than 1x1");
+  using TapBits = std::conditional_t<WIDE, uint64_t, uint32_t>;
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ROWS = VA ? BM / 32 : BM / 8, B_ROWS = VB ? BN / 32 : BN / 8;   // fetches per thread and chunk
   __shared__ __attribute__((aligned(16))) float As[2][BM][kLd];
@@ -132,7 +167,7 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
 
   if (tid < BN) {
     const int j = j0 + tid;
-    int2 e = make_int2(0, BUF ? 31 : (-16384) & 0xffff);   // column beyond J: never valid
+    int2 e = make_int2(0, WIDE ? 63 : BUF ? 31 : (-16384) & 0xffff);   // column beyond J: never valid
     if (j < p.J) {
       const uint32_t c = tt::fd_div((uint32_t)j, p.divRS);
       const uint32_t rs = (uint32_t)j - c * p.divRS.d;
@@ -169,7 +204,8 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   // t is outside the image), and the per-lane constants added per load
   __amdgpu_buffer_rsrc_t dySrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.dy, 0, kSrdRecords, kSrdFlags);
   __amdgpu_buffer_rsrc_t xSrd = __builtin_amdgcn_make_buffer_rsrc((void*)p.x, 0, kSrdRecords, kSrdFlags);
-  uint32_t dyvoff = 0x80000000u, xvoff = 0, nmask = 0xffffffffu;
+  uint32_t dyvoff = 0x80000000u, xvoff = 0;
+  TapBits nmask = ~(TapBits)0;
   int aoff[A_ROWS];
   if constexpr (BUF) {
 #pragma unroll
@@ -189,14 +225,17 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   // chunk ahead so that its latency is covered
   int4 pixnext = make_int4(0, 0, 0, 0);
   int2 pixnextq = make_int2(0, 0);
+  int pixnexthi = 0;
   auto fetch_pix = [&](int chunk) __attribute__((always_inline)) {
     if constexpr (BUF && !(VA && VB)) pixnext = p.pixtab[chunk * kBK + px];
+    if constexpr (WIDE) pixnexthi = p.pixhi[chunk * kBK + px];
     if constexpr (VA || VB) pixnextq = *reinterpret_cast<const int2*>(&p.pixtab[chunk * kBK + 4 * qpx]);
   };
   auto decompose = [&](int chunk, int following) __attribute__((always_inline)) {
     if constexpr (BUF) {
       const int4 e = pixnext;   // entry of `chunk`
       const int2 eq = pixnextq;
+      const int ehi = pixnexthi;
       fetch_pix(following);
       const int n0 = __builtin_amdgcn_readfirstlane((VA && VB) ? eq.x : e.x);   // lane 0 holds the chunk's first pixel
       if constexpr (VA || VB) {
@@ -209,7 +248,8 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
           (void*)(p.x + ((long long)n0 * p.xStrideN + (long long)g * p.xStrideG - p.xBias)), 0, kSrdRecords, kSrdFlags);
       dyvoff = (uint32_t)(4 * (e.x - n0) * p.dyStrideN) + (uint32_t)e.y;   // bit 31 of e.y survives: pixel past the end
       xvoff = (uint32_t)(4 * (e.x - n0) * p.xStrideN) + (uint32_t)e.z;
-      nmask = (uint32_t)e.w;
+      if constexpr (WIDE) nmask = (TapBits)(((uint64_t)(uint32_t)ehi << 32) | (uint32_t)e.w);
+      else nmask = (uint32_t)e.w;
       return;
     }
     const int m = chunk * kBK + px;
@@ -240,7 +280,7 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
           bregv[t] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(xSrd, (int)(qxvoff + (uint32_t)boffv[t]), 0, 0));
         } else {
           const int2 e = jreg[t];
-          const uint32_t vo = ((nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
+          const uint32_t vo = ((uint32_t)(nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
           breg[t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
         }
       }
@@ -428,6 +468,15 @@ template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_bf16(const Wgrad p) {
   wgrad_body<WM, WN, MT, NT, BUF, VA, VB, true>(p);
 }
+// kernels of 32 .. 63 taps: buffer path with 64-bit tap masks
+template <int WM, int WN, int MT, int NT, bool VA>
+__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_wide_f32(const Wgrad p) {
+  wgrad_body<WM, WN, MT, NT, true, VA, false, false, true>(p);
+}
+template <int WM, int WN, int MT, int NT, bool VA>
+__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_wide_bf16(const Wgrad p) {
+  wgrad_body<WM, WN, MT, NT, true, VA, false, true, true>(p);
+}
 
 // dw[e] = sum over splits of partial[s][e] in float64.  A block covers 64 float4 columns with
 // 4 lanes per column; lane l adds splits l, l+4, ... in order, the four lane sums are added in
@@ -485,13 +534,26 @@ struct PixKey {
   }
 };
 // The pixel table depends only on the geometry: built on first use, kept for the process
-// (16 bytes per output pixel; at most kMaxPixTables geometries, then the oldest are dropped).
+// (16 bytes per output pixel, 20 with a 64-bit mask; at most kMaxPixTables geometries, then all are dropped).
 constexpr size_t kMaxPixTables = 256;
-std::map<PixKey, int4*>& pixtab_cache() {
-  static std::map<PixKey, int4*> cache;
+struct PixTables {
+  int4* tab;
+  int* hi;   // null unless the kernel has 32 .. 63 taps
+};
+std::map<PixKey, PixTables>& pixtab_cache() {
+  static std::map<PixKey, PixTables> cache;
   return cache;
 }
-int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
+int drop_pixtabs() {
+  auto& cache = pixtab_cache();
+  for (auto& kv : cache) {
+    TT_HIP(hipFree(kv.second.tab));
+    if (kv.second.hi) TT_HIP(hipFree(kv.second.hi));
+  }
+  cache.clear();
+  return 0;
+}
+int cached_pixtab(const Wgrad& p, int N, int P, int Q, bool wide, const int4** out, const int** out_hi) {
   auto& cache = pixtab_cache();
   const PixKey key{{N, P, Q, p.H, p.W, p.sh, p.sw, p.ph, p.pw, p.dh, p.dw, p.R, p.S, p.chunks}};
   auto it = cache.find(key);
@@ -499,25 +561,40 @@ int cached_pixtab(const Wgrad& p, int N, int P, int Q, const int4** out) {
     hipStream_t st = tt::stream();
     if (cache.size() >= kMaxPixTables) {
       TT_HIP(hipStreamSynchronize(st));
-      for (auto& kv : cache) TT_HIP(hipFree(kv.second));
-      cache.clear();
+      if (drop_pixtabs()) return -1;
     }
     const int entries = p.chunks * kBK;
-    int4* tab = nullptr;
-    TT_HIP(hipMalloc((void**)&tab, sizeof(int4) * (size_t)entries));
-    wgrad_build_pixtab<<<ceil_div(entries, 256), 256, 0, st>>>(tab, p, entries, N);
+    PixTables t{nullptr, nullptr};
+    TT_HIP(hipMalloc((void**)&t.tab, sizeof(int4) * (size_t)entries));
+    if (wide) {
+      if (hipError_t e = hipMalloc((void**)&t.hi, sizeof(int) * (size_t)entries); e != hipSuccess) {
+        (void)hipFree(t.tab);
+        return tt::fail_hip(e, "hipMalloc", __FILE__, __LINE__);
+      }
+    }
+    wgrad_build_pixtab<<<ceil_div(entries, 256), 256, 0, st>>>(t.tab, t.hi, p, entries, N);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) {
-      (void)hipFree(tab);
+      (void)hipFree(t.tab);
+      if (t.hi) (void)hipFree(t.hi);
       return tt::fail_hip(e, "wgrad_build_pixtab", __FILE__, __LINE__);
     }
-    it = cache.emplace(key, tab).first;
+    it = cache.emplace(key, t).first;
   }
-  *out = it->second;
+  *out = it->second.tab;
+  *out_hi = it->second.hi;
   return 0;
 }
 
 template <int WM, int WN, int MT, int NT>
-void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStream_t st) {
+void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, bool wide, hipStream_t st) {
+  if (wide) {   // implies buf and not vb
+    const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
+    if (bf && va) wgrad_wide_bf16<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
+    else if (bf) wgrad_wide_bf16<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
+    else if (va) wgrad_wide_f32<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
+    else wgrad_wide_f32<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
+    return;
+  }
   if (tt::conv_math() == TT_CONV_MATH_BF16) {
     if (buf && va && vb) wgrad_bf16<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
     else if (buf && va) wgrad_bf16<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
@@ -535,10 +612,7 @@ void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, hipStre
 
 namespace tt {
 int wgrad_release_tables() {   // the caller has synchronised the stream
-  auto& cache = pixtab_cache();
-  for (auto& kv : cache) TT_HIP(hipFree(kv.second));
-  cache.clear();
-  return 0;
+  return drop_pixtabs();
 }
 }  // namespace tt
 
@@ -640,8 +714,9 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     // (a chunk spans at most 33 images; x offsets also carry the column's tap and channel offset)
     const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
                                  ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
-    const bool buf = R * S <= 31 && reach < (1LL << 31) - (1LL << 20);
-    if (buf && cached_pixtab(p, r.n, P, Q, &p.pixtab)) return -1;
+    const bool buf = R * S <= 63 && reach < (1LL << 31) - (1LL << 20);
+    const bool wide = buf && R * S > 31;
+    if (buf && cached_pixtab(p, r.n, P, Q, wide, &p.pixtab, &p.pixhi)) return -1;
     // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
     const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)p.dy & 15) == 0;
     const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)p.x & 15) == 0;
@@ -649,13 +724,13 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     {
       tt::ProfScope prof(TT_PROF_CONV_WGRAD);
       if (bm == 128 && bn == 128)
-        launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, st);
+        launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, wide, st);
       else if (bm == 64 && bn == 128)
-        launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, st);
+        launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, wide, st);
       else if (bm == 128 && bn == 64)
-        launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, st);
+        launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, wide, st);
       else
-        launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, st);
+        launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, wide, st);
     }
     TT_LAUNCH_CHECK();
   }

@@ -77,7 +77,11 @@ TILE_CASES = [
     (3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2),         # plain-GEMM path with groups, ragged pixel tile
     (70, 16, 3, 3, 32, 3, 3, (1, 1), (1, 1), (1, 1), 1),        # tiny images: a pixel tile spans 15-29 images (buffer re-basing)
     (5, 32, 13, 9, 48, 5, 5, (2, 1), (4, 2), (2, 1), 2),        # 25 taps, dilation + stride + groups: tap masks, negative table steps in dgrad
-    (3, 16, 14, 14, 16, 6, 6, (1, 1), (2, 2), (1, 1), 1),       # 36 taps > 31: compare-and-select addressing in all three passes
+    (3, 16, 14, 14, 16, 6, 6, (1, 1), (2, 2), (1, 1), 1),       # 36 taps > 31: 64-bit tap masks in forward and weight gradient, compare-and-select in the input gradient
+    (2, 8, 20, 18, 24, 7, 9, (1, 1), (3, 4), (1, 1), 1),        # 63 taps: the most a 64-bit tap mask holds (its top bit is the padding tap)
+    (4, 6, 23, 25, 40, 7, 7, (2, 2), (3, 3), (1, 1), 2),        # 49 taps with groups, stride 2 and an odd image
+    (2, 4, 30, 30, 16, 6, 7, (1, 2), (5, 6), (2, 2), 1),        # 42 taps with dilation 2 and padding wider than the kernel's reach on one side
+    (3, 16, 14, 14, 16, 9, 9, (1, 1), (4, 4), (1, 1), 1),       # 81 taps > 63: compare-and-select addressing in all three passes
     (2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1),       # padded 1x1: not the plain-GEMM geometry, one-tap mask
     (4, 48, 10, 10, 24, 3, 3, (1, 1), (0, 0), (1, 1), 1),       # unpadded 3x3, rows (24) and weight rows shorter than a tile
     (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)
@@ -101,7 +105,7 @@ TILE_CASES = [
 
 def test_tile_case_list_is_complete():
     """A case that slips into the comment of the line above it would silently drop out."""
-    assert len(TILE_CASES) == 36
+    assert len(TILE_CASES) == 40
     assert all(len(c) == 11 for c in TILE_CASES)
     strided_1x1 = [c for c in TILE_CASES if c[5:7] == (1, 1) and c[7] != (1, 1) and c[10] == 1]
     assert {c[7][0] for c in strided_1x1} == {2, 3, 4}      # cells two, three and four rows high
