@@ -58,8 +58,9 @@ __device__ __forceinline__ double wave_sum(double v) {
   return readlane_d(v, 0) + readlane_d(v, 32);
 }
 
-// Two sums per block: wave_sum, then the four waves through LDS.  Result valid in all threads.
-__device__ __forceinline__ void block_sum2(double& a, double& b, double* lds /* 2*kWaves */) {
+// Two sums per block: wave_sum, then the waves through LDS in wave order.  Result valid in all threads.
+template <int WAVES = kWaves>
+__device__ __forceinline__ void block_sum2(double& a, double& b, double* lds /* 2*WAVES */) {
   a = wave_sum(a);
   b = wave_sum(b);
   const int wave = threadIdx.x >> 6;
@@ -71,7 +72,7 @@ __device__ __forceinline__ void block_sum2(double& a, double& b, double* lds /* 
   a = 0;
   b = 0;
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) {
+  for (int w = 0; w < WAVES; ++w) {
     a += lds[2 * w];
     b += lds[2 * w + 1];
   }
@@ -506,19 +507,23 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_apply(BwdArgs a, Geometry g) 
 }
 
 // ---- small channels: one kernel per pass ---------------------------------------------------------
-// When a channel's N*HW values fit the registers of one block (<= kThreads * EMAX), the block
+// When a channel's N*HW values fit the registers of one block (<= BT * EMAX, BT threads), the block
 // reads them once, reduces, and applies from registers: S read + S written forward, 2S + S
 // backward instead of 3S and 5S, and one launch instead of two.  Grid = C blocks; g.hwv_div
 // divides by HW.  The deep layers of a network (7x7 to 16x16 planes, hundreds of channels) are
 // of this kind.  Statistics and coefficients follow the two-sweep kernels' formulas exactly.
+// Larger channels take 64 values per thread, or -- when there are so few channels that a CU gets
+// two blocks at most -- blocks of 1024 threads with 16 values each: more waves on a CU keep loads
+// in flight while others reduce or store (measured, 256 channels of 64 x 14 x 14 values: backward
+// 32 -> 15 us, forward 12.5 -> 10 us; 1024 such channels are 10 % slower that way and keep 256 threads).
 
-template <int EMAX, typename F>
+template <int EMAX, int BT, typename F>
 __device__ __forceinline__ void for_channel_elements(const Geometry& g, F&& f) {
   const int total = g.N * g.HW;
   const size_t image = (size_t)g.C * g.HW;
 #pragma unroll
   for (int k = 0; k < EMAX; ++k) {
-    const int e = (int)threadIdx.x + k * kThreads;
+    const int e = (int)threadIdx.x + k * BT;
     if (e < total) {
       const uint32_t n = tt::fd_div((uint32_t)e, g.hwv_div);
       f(k, (size_t)n * image + ((uint32_t)e - n * (uint32_t)g.HW));
@@ -526,23 +531,23 @@ __device__ __forceinline__ void for_channel_elements(const Geometry& g, F&& f) {
   }
 }
 
-template <int EMAX, bool kRelu = false>
-__global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) {
-  __shared__ double red[2 * kWaves];
+template <int EMAX, int BT, bool kRelu = false>
+__global__ __launch_bounds__(BT) void bn_fwd_small(FwdArgs a, Geometry g) {
+  __shared__ double red[2 * BT / tt::kWave];
   __shared__ Coef sk;
   const int c = blockIdx.x;
   const float* __restrict__ xc = a.x + (size_t)c * g.HW;
   float* __restrict__ yc = a.y + (size_t)c * g.HW;
   const float shift = xc[0];
   float v[EMAX];
-  for_channel_elements<EMAX>(g, [&](int k, size_t off) { v[k] = xc[off]; });
+  for_channel_elements<EMAX, BT>(g, [&](int k, size_t off) { v[k] = xc[off]; });
   double s1 = 0.0, s2 = 0.0;
-  for_channel_elements<EMAX>(g, [&](int k, size_t) {
+  for_channel_elements<EMAX, BT>(g, [&](int k, size_t) {
     const double d = (double)(v[k] - shift);
     s1 += d;
     s2 += d * d;
   });
-  block_sum2(s1, s2, red);
+  block_sum2<BT / tt::kWave>(s1, s2, red);
   if (threadIdx.x == 0) {
     const double m = (double)g.N * (double)g.HW;
     const double d1 = s1 / m;
@@ -565,32 +570,32 @@ __global__ __launch_bounds__(kThreads) void bn_fwd_small(FwdArgs a, Geometry g) 
   }
   __syncthreads();
   const Coef k = sk;
-  for_channel_elements<EMAX>(g, [&](int kk, size_t off) {
+  for_channel_elements<EMAX, BT>(g, [&](int kk, size_t off) {
     const float o = fmaf(v[kk] - k.m, k.k1, k.k0);
     __builtin_nontemporal_store(kRelu ? relu1(o) : o, yc + off);
   });
 }
 
-template <int EMAX, bool kRelu = false>
-__global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) {
-  __shared__ double red[2 * kWaves];
+template <int EMAX, int BT, bool kRelu = false>
+__global__ __launch_bounds__(BT) void bn_bwd_small(BwdArgs a, Geometry g) {
+  __shared__ double red[2 * BT / tt::kWave];
   __shared__ Coef sk;
   const int c = blockIdx.x;
   const float* __restrict__ xc = a.x + (size_t)c * g.HW;
   const float* __restrict__ dyc = a.dy + (size_t)c * g.HW;
   const float mean = a.save_mean[c];
   float v[EMAX], gq[EMAX];
-  for_channel_elements<EMAX>(g, [&](int k, size_t off) {
+  for_channel_elements<EMAX, BT>(g, [&](int k, size_t off) {
     v[k] = __builtin_nontemporal_load(xc + off);
     gq[k] = __builtin_nontemporal_load(dyc + off);
     if constexpr (kRelu) gq[k] = mask1(gq[k], __builtin_nontemporal_load(a.ry + (size_t)c * g.HW + off));
   });
   double s_dy = 0.0, s_dyxmu = 0.0;
-  for_channel_elements<EMAX>(g, [&](int k, size_t) {
+  for_channel_elements<EMAX, BT>(g, [&](int k, size_t) {
     s_dy += (double)gq[k];
     s_dyxmu += (double)gq[k] * (double)(v[k] - mean);
   });
-  block_sum2(s_dy, s_dyxmu, red);
+  block_sum2<BT / tt::kWave>(s_dy, s_dyxmu, red);
   if (threadIdx.x == 0) {
     const double m = (double)g.N * (double)g.HW;
     const double sd = (double)a.save_sd[c];
@@ -607,7 +612,7 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) 
   __syncthreads();
   const Coef k = sk;
   float* __restrict__ dxc = a.dx + (size_t)c * g.HW;
-  for_channel_elements<EMAX>(g, [&](int kk, size_t off) {
+  for_channel_elements<EMAX, BT>(g, [&](int kk, size_t off) {
     __builtin_nontemporal_store(fmaf(gq[kk], k.k1, fmaf(v[kk] - k.m, k.k2, k.k0)), dxc + off);
   });
 }
@@ -617,11 +622,14 @@ __global__ __launch_bounds__(kThreads) void bn_bwd_small(BwdArgs a, Geometry g) 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
 // Channels small enough for the single-kernel passes, and enough of them to fill the device.
-constexpr int kSmallMax = 64;   // values per thread
-int small_channel_capacity(int N, int C, int HW) {
+constexpr int kSmallValues = 16, kSmallValuesMax = 64;   // values per thread
+constexpr int kSmallThreads = 1024;                     // threads of the larger block size
+// 0: two-sweep kernels; 1: 256 threads x 16 values; 2: 256 x 64; 3: 1024 x 16
+int small_channel_config(int N, int C, int HW) {
   const long long total = (long long)N * HW;
-  if (C < 128 || total > (long long)kThreads * kSmallMax) return 0;
-  return total <= (long long)kThreads * 16 ? 16 : kSmallMax;
+  if (C < 128 || total > (long long)kThreads * kSmallValuesMax) return 0;
+  if (total <= (long long)kThreads * kSmallValues) return 1;
+  return C <= 2 * tt::compute_units() ? 3 : 2;
 }
 Geometry small_geometry(int N, int C, int HW) {
   Geometry g{};
@@ -777,15 +785,17 @@ static int bn_fwd_train(const char* fn, const float* x, const float* gamma, cons
   a.unbias = (float)((double)m / (double)(m - 1));
   a.eps = (float)eps;
   hipStream_t st = tt::stream();
-  if (const int cap = small_channel_capacity(N, C, HW)) {
+  if (const int cfg = small_channel_config(N, C, HW)) {
     tt::ProfScope prof(timed ? TT_PROF_BN_FWD_APPLY : -1);
     const Geometry gs = small_geometry(N, C, HW);
     if (relu) {
-      if (cap == 16) bn_fwd_small<16, true><<<C, kThreads, 0, st>>>(a, gs);
-      else bn_fwd_small<kSmallMax, true><<<C, kThreads, 0, st>>>(a, gs);
+      if (cfg == 1) bn_fwd_small<kSmallValues, kThreads, true><<<C, kThreads, 0, st>>>(a, gs);
+      else if (cfg == 2) bn_fwd_small<kSmallValuesMax, kThreads, true><<<C, kThreads, 0, st>>>(a, gs);
+      else bn_fwd_small<kSmallValues, kSmallThreads, true><<<C, kSmallThreads, 0, st>>>(a, gs);
     } else {
-      if (cap == 16) bn_fwd_small<16><<<C, kThreads, 0, st>>>(a, gs);
-      else bn_fwd_small<kSmallMax><<<C, kThreads, 0, st>>>(a, gs);
+      if (cfg == 1) bn_fwd_small<kSmallValues, kThreads><<<C, kThreads, 0, st>>>(a, gs);
+      else if (cfg == 2) bn_fwd_small<kSmallValuesMax, kThreads><<<C, kThreads, 0, st>>>(a, gs);
+      else bn_fwd_small<kSmallValues, kSmallThreads><<<C, kSmallThreads, 0, st>>>(a, gs);
     }
     TT_LAUNCH_CHECK();
     return 0;
@@ -899,17 +909,19 @@ static int bn_bwd(const char* fn, const float* x, const float* dy, const float* 
   TT_REQUIRE(x && dy && save_mean && save_var_eps && save_sd, "%s: null tensor pointer", fn);
   TT_REQUIRE_ALIGNED(fn, x, dy, dx, ry);
   if (!dx && !dgamma && !dbeta) return 0;
-  if (const int cap = small_channel_capacity(N, C, HW)) {
+  if (const int cfg = small_channel_config(N, C, HW)) {
     tt::ProfScope prof(TT_PROF_BN_BWD_APPLY);
     const Geometry gs = small_geometry(N, C, HW);
     BwdArgs b{x, dy, gamma, save_mean, save_var_eps, save_sd, dx, dgamma, dbeta, nullptr, 0, ry};
     hipStream_t st = tt::stream();
     if (ry) {
-      if (cap == 16) bn_bwd_small<16, true><<<C, kThreads, 0, st>>>(b, gs);
-      else bn_bwd_small<kSmallMax, true><<<C, kThreads, 0, st>>>(b, gs);
+      if (cfg == 1) bn_bwd_small<kSmallValues, kThreads, true><<<C, kThreads, 0, st>>>(b, gs);
+      else if (cfg == 2) bn_bwd_small<kSmallValuesMax, kThreads, true><<<C, kThreads, 0, st>>>(b, gs);
+      else bn_bwd_small<kSmallValues, kSmallThreads, true><<<C, kSmallThreads, 0, st>>>(b, gs);
     } else {
-      if (cap == 16) bn_bwd_small<16><<<C, kThreads, 0, st>>>(b, gs);
-      else bn_bwd_small<kSmallMax><<<C, kThreads, 0, st>>>(b, gs);
+      if (cfg == 1) bn_bwd_small<kSmallValues, kThreads><<<C, kThreads, 0, st>>>(b, gs);
+      else if (cfg == 2) bn_bwd_small<kSmallValuesMax, kThreads><<<C, kThreads, 0, st>>>(b, gs);
+      else bn_bwd_small<kSmallValues, kSmallThreads><<<C, kSmallThreads, 0, st>>>(b, gs);
     }
     TT_LAUNCH_CHECK();
     return 0;
@@ -980,7 +992,7 @@ int tt_channel_sum_f32(const float* t, float* out, int N, int K, int HW) {
 int tt_workspace_size_bn_f32(size_t* bytes, int N, int C, int HW) {
   TT_REQUIRE(bytes, "tt_workspace_size_bn_f32: null result pointer");
   if (check_shape("tt_workspace_size_bn_f32", N, C, HW)) return -1;
-  if (small_channel_capacity(N, C, HW)) {   // single-kernel passes: no partials
+  if (small_channel_config(N, C, HW)) {   // single-kernel passes: no partials
     *bytes = 0;
     return 0;
   }

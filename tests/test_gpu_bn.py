@@ -235,8 +235,11 @@ def test_bn_random_shapes(shape):
 # at least 128 channels of at most 16384 values each: the single-kernel passes (one block per channel
 # keeps the channel in registers); the last two sit just inside and just outside that limit
 SMALL_CHANNEL_SHAPES = [
-    (64, 256, 7, 7),      # 3136 values: 16 per thread
-    (32, 128, 14, 14),    # 6272 values: 64-per-thread instance, partly filled
+    (64, 256, 7, 7),      # 3136 values: 256 threads x 16 values
+    (32, 128, 14, 14),    # 6272 values, few channels: 1024 threads x 16 values, partly filled
+    (64, 256, 14, 14),    # 12544 values, 256 channels (ResNet-50's 14x14 stage): 1024 threads x 16
+    (16, 640, 20, 20),    # 6400 values, more channels than two blocks per CU: 256 threads x 64 values
+    (64, 1024, 14, 14),   # the same at ResNet-50's size
     (2, 128, 1, 1),       # two values per channel
     (3, 200, 5, 7),       # odd plane, threads without a value
     (128, 512, 4, 4),     # DCGAN / PreAct-ResNet-18 deepest layers

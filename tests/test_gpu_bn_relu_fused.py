@@ -20,9 +20,10 @@ import oracle
 pytestmark = pytest.mark.gpu
 
 # two-sweep kernels: plane mode, flat float4, flat scalar, stream reduce with several splits;
-# single-kernel path for small channels (16 and 64 values per thread)
+# single-kernel path for small channels (256 threads x 16 values, 1024 x 16 with few channels, 256 x 64 with many)
 SHAPES = [(4, 3, 5, 5), (16, 5, 4, 4), (8, 64, 14, 14), (6, 16, 16, 16), (5, 7, 24, 20), (64, 64, 28, 28),
-          (128, 4, 32, 32), (96, 12, 28, 28), (4, 128, 7, 7), (8, 256, 14, 14), (16, 130, 9, 7)]
+          (128, 4, 32, 32), (96, 12, 28, 28), (4, 128, 7, 7), (8, 256, 14, 14), (16, 130, 9, 7),
+          (32, 256, 14, 14), (24, 576, 14, 14)]
 
 
 def _bits_equal(a, b, name):
