@@ -535,7 +535,9 @@ template <int EMAX, int BT, bool kRelu = false>
 __global__ __launch_bounds__(BT) void bn_fwd_small(FwdArgs a, Geometry g) {
   __shared__ double red[2 * BT / tt::kWave];
   __shared__ Coef sk;
-  const int c = blockIdx.x;
+  // neighbouring channels share cache lines wherever a plane is not a whole number of lines (7x7: 196
+  // bytes): blocks of one die (every eighth block of the grid) take a contiguous run of channels
+  const int c = tt::xcd_remap((int)blockIdx.x, (int)gridDim.x);
   const float* __restrict__ xc = a.x + (size_t)c * g.HW;
   float* __restrict__ yc = a.y + (size_t)c * g.HW;
   const float shift = xc[0];
@@ -580,7 +582,9 @@ template <int EMAX, int BT, bool kRelu = false>
 __global__ __launch_bounds__(BT) void bn_bwd_small(BwdArgs a, Geometry g) {
   __shared__ double red[2 * BT / tt::kWave];
   __shared__ Coef sk;
-  const int c = blockIdx.x;
+  // neighbouring channels share cache lines wherever a plane is not a whole number of lines (7x7: 196
+  // bytes): blocks of one die (every eighth block of the grid) take a contiguous run of channels
+  const int c = tt::xcd_remap((int)blockIdx.x, (int)gridDim.x);
   const float* __restrict__ xc = a.x + (size_t)c * g.HW;
   const float* __restrict__ dyc = a.dy + (size_t)c * g.HW;
   const float mean = a.save_mean[c];
