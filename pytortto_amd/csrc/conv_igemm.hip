@@ -397,7 +397,7 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   };
   auto load_a_item = [&](int chunk, int it) __attribute__((always_inline)) {
     const int q = aq0 + it * (kThreads / BM);   // always < kBKQ unless the tile has fewer than 64 rows
-    if (q < kBKQ) {
+    if (BM >= 64 || q < kBKQ) {   // (the compile-time half keeps the load out of a divergent branch)
       const int kq = chunk * kBKQ + q;
       if constexpr (AT) {
         // four k values of this row: one coalesced dword load each (whole chunks only)
@@ -433,7 +433,7 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   };
   auto store_a_item = [&](int buf, int it) __attribute__((always_inline)) {
     const int q = aq0 + it * (kThreads / BM);
-    if (q < kBKQ) As[buf][q][arow] = areg[it];
+    if (BM >= 64 || q < kBKQ) As[buf][q][arow] = areg[it];
   };
   auto store_b_item = [&](int buf, int it) __attribute__((always_inline)) {
     floatx4 v = breg[it];
