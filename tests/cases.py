@@ -82,6 +82,29 @@ def random_conv_cases(count, seed):
     return cases
 
 
+def random_large_kernel_cases(count, seed):
+    """Seeded random geometries with kernels of 26 to 81 taps: beyond a 32-bit tap mask (31 taps) the
+    device kernels keep 64-bit masks, beyond 63 taps they compare bounds per element."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        g = int(rng.choice([1, 1, 2]))
+        c, k = g * int(rng.integers(1, 12)), g * int(rng.integers(1, 20))
+        r, s = int(rng.integers(3, 10)), int(rng.integers(3, 10))
+        if r * s < 26:
+            continue
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pd = (int(rng.integers(0, 6)), int(rng.integers(0, 6)))
+        h, w = int(rng.integers(6, 30)), int(rng.integers(6, 30))
+        n = int(rng.integers(1, 5))
+        if h + 2 * pd[0] < dl[0] * (r - 1) + 1 or w + 2 * pd[1] < dl[1] * (s - 1) + 1:
+            continue
+        cases.append((n, c, h, w, k, r, s, st, pd, dl, g))
+    return cases
+
+
 def random_convt_cases(count, seed):
     """Seeded random transposed-convolution geometries with output_padding < stride: what the
     reference's own `output_size` path can produce (nn/modules/conv.py:137-153); beyond that its

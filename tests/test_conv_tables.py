@@ -13,7 +13,7 @@ import ctypes
 
 import pytest
 
-from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases, random_large_kernel_cases
 
 
 def _lib():
@@ -107,6 +107,8 @@ def test_tables_of_random_geometries(seed):
         _check_conv(case)
     for case in random_convt_cases(100, seed):
         _check_convt(case)
+    for case in random_large_kernel_cases(100, seed):   # 64-bit tap masks, and the fall-back beyond 63 taps
+        _check_conv(case)
 
 
 def test_table_check_reports_unsupported_geometries_instead_of_tables():

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle
-from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
+from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases, random_large_kernel_cases
 
 pytestmark = pytest.mark.gpu
 
@@ -210,6 +210,14 @@ def test_conv_rejects_bad_arguments():
     c[0], c[1], c[2], c[3], c[4], c[5], c[6], '%d%d' % c[7], '%d%d' % c[8], '%d%d' % c[9], c[10]))
 def test_conv_random_geometries(case):
     _run_conv(case, seed=5)
+
+
+@pytest.mark.parametrize('case', random_large_kernel_cases(40, 99), ids=lambda c: 'n%d_c%d_%dx%d_k%d_%dx%d_s%s_p%s_d%s_g%d' % (
+    c[0], c[1], c[2], c[3], c[4], c[5], c[6], '%d%d' % c[7], '%d%d' % c[8], '%d%d' % c[9], c[10]))
+def test_conv_random_large_kernels(case):
+    """Kernels of 26 to 81 taps with random stride, padding, dilation and groups: 32-bit tap masks,
+    64-bit tap masks (32 to 63 taps) and per-element bounds (more than 63) in all three passes."""
+    _run_conv(case, seed=6)
 
 
 @pytest.mark.parametrize('case', [
