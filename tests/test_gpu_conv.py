@@ -82,6 +82,7 @@ TILE_CASES = [
     (4, 6, 23, 25, 40, 7, 7, (2, 2), (3, 3), (1, 1), 2),        # 49 taps with groups, stride 2 and an odd image
     (2, 4, 30, 30, 16, 6, 7, (1, 2), (5, 6), (2, 2), 1),        # 42 taps with dilation 2 and padding wider than the kernel's reach on one side
     (3, 16, 14, 14, 16, 9, 9, (1, 1), (4, 4), (1, 1), 1),       # 81 taps > 63: compare-and-select addressing in all three passes
+    (2, 2, 20, 22, 4, 13, 11, (2, 2), (6, 5), (1, 1), 1),       # few channels, stride 2, 13x11 kernel: the dense input gradient's union window has 7x6 = 42 taps (64-bit masks there too)
     (2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1),       # padded 1x1: not the plain-GEMM geometry, one-tap mask
     (4, 48, 10, 10, 24, 3, 3, (1, 1), (0, 0), (1, 1), 1),       # unpadded 3x3, rows (24) and weight rows shorter than a tile
     (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),         # C*R*S = 180: weight rows not a whole number of 16-wide chunks (repacked copy)
@@ -105,7 +106,7 @@ TILE_CASES = [
 
 def test_tile_case_list_is_complete():
     """A case that slips into the comment of the line above it would silently drop out."""
-    assert len(TILE_CASES) == 40
+    assert len(TILE_CASES) == 41
     assert all(len(c) == 11 for c in TILE_CASES)
     strided_1x1 = [c for c in TILE_CASES if c[5:7] == (1, 1) and c[7] != (1, 1) and c[10] == 1]
     assert {c[7][0] for c in strided_1x1} == {2, 3, 4}      # cells two, three and four rows high
