@@ -507,6 +507,13 @@ def main():
             for _ in range(l.count):
                 l.run(call)
 
+    # ---- what the device sustains on the two bounding resources, measured in this run ----------
+    # (first: 0.2 s of dense matrix work and 8 GiB of streaming also bring the device from idle to
+    # its sustained clocks before anything is timed; with 3 warm-up steps alone the first timed
+    # steps still run on the ramp)
+    mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
+    hbm_read, hbm_copy = _hip.probe_hbm(2 << 30)
+
     conv_ms, conv_wall_ms = timed_steps(_hip, conv_step, args.steps, args.warmup)
     conv_tflops = 3 * flops_per_pass / (conv_ms * 1e-3) / 1e12
     prof = profiled_steps(_hip, conv_step, args.steps)
@@ -653,10 +660,6 @@ def main():
                       'conv_tflops_equivalent': round(3 * 26.78e9 / (d_wall * 1e-3) / 1e12, 2)},
                   'note': 'whole stacks, every kernel counted in the time, only convolution FLOPs in the rate; '
                           'the input of the first layer needs no gradient, so its input-gradient pass does not run'}
-
-    # ---- what the device sustains on the two bounding resources, measured in this run ----------
-    mfma_mean, mfma_min, mfma_max = _hip.probe_mfma(100)
-    hbm_read, hbm_copy = _hip.probe_hbm(2 << 30)
 
     # ---- CPU baseline (oracle on the host cores) -------------------------------------------------
     cpu_conv = cpu_bn = None
