@@ -116,9 +116,9 @@ int tt_get_conv_math(int* mode);   /* host pointer */
  * Such launches stack the pixel classes of a cell of the output (one period of the stride
  * pattern, or two / four periods side by side) as rows of one matrix product; a larger cell
  * wastes fewer multiplications but leaves fewer tiles.  A larger cell is taken only while at
- * least `tiles` tiles of 256 cells remain (default 384 = 1.5 per compute unit; 0 = always, which
- * lets small inputs reach the larger cells).  Results do not depend on it beyond summation
- * order.  Process-wide, applies to later calls. */
+ * least `tiles` tiles of 256 cells remain (default 1.5 per compute unit, 384 on an MI355X; 0 =
+ * always, which lets small inputs reach the larger cells; -1 = back to the default).  Results do
+ * not depend on it beyond summation order.  Process-wide, applies to later calls. */
 int tt_set_conv_dense_cell_min_tiles(int tiles);
 
 /* y[N,K,P,Q] = conv(x[N,C,H,W], w[K,C/groups,R,S]) (+ bias[K] if not NULL).
@@ -143,13 +143,17 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
 /* dw[K,C/groups,R,S] = sum over n,p,q of x~[n,c,p*sh+r*dh-ph,q*sw+s*dw-pw] * dy[n,k,p,q]
  * (x~ = x zero-padded).  Deterministic: fixed split of the reduction, partial sums combined
  * in float64.  Replaces _conv2d_backward_w: autograd/grad_nn.py:646-656 (called from :731
- * and, with the roles of x and dy exchanged by the caller, :776). */
+ * and, with the roles of x and dy exchanged by the caller, :776).
+ * P, Q are the spatial size of dy; they may be smaller than the geometry's output size (the
+ * reference crops x~ to the rows the windows cover, :653-655) but not larger: a dy that does not
+ * belong to the geometry is refused. */
 int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw,
                         int N, int C, int H, int W, int K, int R, int S,
                         int sh, int sw, int ph, int pw, int dh, int dw_, int groups,
                         int P, int Q);
 
-/* Host-only checks of the index tables behind tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 (no
+/* Host-only checks of the index tables behind tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 /
+ * tt_conv2d_wgrad_f32 (no
  * counterpart in the reference; no device is needed and tt_init() need not have been called).
  * The kernels turn a reduction index (c, r, s) -- (k, tap row, tap column) for the input gradient
  * -- into an address through small per-geometry tables, which the library builds on the host,
@@ -157,14 +161,47 @@ int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw,
  * that planning and check for a geometry without launching anything: every table entry, replayed
  * for the extreme pixels under the kernel's own bounds rule, must address the element of x (dy)
  * that autograd/grad_nn.py:603-611 (:659-682) pairs with that reduction index, inside the tensor.
- * tt_conv2d_check_tables_selftest damages single entries and returns 0 when the check refuses each
- * damaged table. */
+ * The weight gradient's table has one entry per output pixel (image, offsets of the pixel in dy
+ * and of its window in x, one bit per tap that falls into the padding); every entry is checked:
+ * the dy element and, tap by tap, the x element it leads to must be the ones
+ * autograd/grad_nn.py:646-656 pairs, inside the tensors, and a tap is blocked exactly when it lies
+ * in the padding.
+ * tt_conv2d_check_tables_selftest / _selftest_wgrad damage single entries and return 0 when the
+ * check refuses each damaged table. */
 int tt_conv2d_check_tables_fwd_f32(int N, int C, int H, int W, int K, int R, int S,
                                    int sh, int sw, int ph, int pw, int dh, int dw, int groups);
 int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R, int S,
                                      int sh, int sw, int ph, int pw, int dh, int dw, int groups,
                                      int P, int Q);
+int tt_conv2d_check_tables_wgrad_f32(int N, int C, int H, int W, int K, int R, int S,
+                                     int sh, int sw, int ph, int pw, int dh, int dw_, int groups,
+                                     int P, int Q);
 int tt_conv2d_check_tables_selftest(void);
+int tt_conv2d_check_tables_selftest_wgrad(void);
+
+/* Instrumentation of the convolution launches (tests only; no counterpart in the reference).
+ * Layers whose tile count loads the compute units unevenly run as one persistent grid of two
+ * blocks per compute unit (three with bf16 arithmetic) whose blocks hand partial sums to each
+ * other; that is safe only while the whole grid is resident, so the library asks the device how
+ * many blocks of each such kernel a compute unit holds and launches one tile per block instead
+ * where it is too few.
+ *   tt_conv2d_stream_k_blocks_per_cu: the smallest answer over all such kernels (host pointer).
+ *   tt_conv2d_stream_k_force_occupancy: pretend the answer is `blocks` (-1: ask the device).
+ *   tt_conv2d_selftest_raise_async_error: a one-thread kernel sets the word that a block sets when
+ *     its bounded wait for another block runs out; the next tt_sync() / tt_memcpy_d2h() returns
+ *     the error, once.  Nothing waits and nothing fails on the device.
+ *   tt_conv2d_images_per_run (host-only): images per run when a batch of N images of image_a
+ *     (input) and image_b (output) elements is cut into runs below 2^31 elements; every run starts
+ *     16-byte aligned; 0 = impossible (the call itself then returns an error). */
+int tt_conv2d_stream_k_blocks_per_cu(int bf16, int* blocks);
+int tt_conv2d_stream_k_force_occupancy(int blocks);
+int tt_conv2d_selftest_raise_async_error(void);
+int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* per);
+/* The plan of the last single matrix-product launch made by tt_conv2d_fwd_f32 / _dgrad_f32 (host
+ * pointer to 8 ints): tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent
+ * grid (0 = one tile per block), tiles computed whole, blocks sharing the remaining tiles'
+ * reductions, addressing mode.  Tests use it to compare the images where the shared tiles begin. */
+int tt_conv2d_last_launch(int* plan8);
 
 /* out[K] = sum over n and the HW plane of t[N,K,HW]: the bias gradient gd0.sum((0,2,3)),
  * autograd/grad_nn.py:728, :774. */

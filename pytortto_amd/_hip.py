@@ -6,6 +6,7 @@ CPU fallback behind this module.
 """
 import ctypes
 import os
+import threading
 from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_void_p
 
 from ._paths import LIB_PATH
@@ -42,7 +43,14 @@ PROTOTYPES = {
     'tt_conv2d_wgrad_f32': [_P, _P, _P] + [_I] * 16,
     'tt_conv2d_check_tables_fwd_f32': [_I] * 14,
     'tt_conv2d_check_tables_dgrad_f32': [_I] * 16,
+    'tt_conv2d_check_tables_wgrad_f32': [_I] * 16,
     'tt_conv2d_check_tables_selftest': [],
+    'tt_conv2d_check_tables_selftest_wgrad': [],
+    'tt_conv2d_stream_k_blocks_per_cu': [_I, POINTER(c_int)],
+    'tt_conv2d_stream_k_force_occupancy': [_I],
+    'tt_conv2d_selftest_raise_async_error': [],
+    'tt_conv2d_last_launch': [POINTER(c_int)],
+    'tt_conv2d_images_per_run': [_I, ctypes.c_longlong, ctypes.c_longlong, POINTER(c_int)],
     'tt_channel_sum_f32': [_P, _P, _I, _I, _I],
     'tt_workspace_size_conv2d_fwd_f32': [POINTER(c_size_t)] + [_I] * 14,
     'tt_workspace_size_conv2d_dgrad_f32': [POINTER(c_size_t)] + [_I] * 16,
@@ -120,18 +128,25 @@ def lib():
 # ---- one deferred operation ----------------------------------------------------------------------
 # An operation whose result the very next operation may absorb (BatchNorm's normalisation into a
 # following ReLU, a ReLU's gradient mask into the BatchNorm backward behind it) is not launched at
-# once: its caller parks it here.  The next operation either takes it over (``take_pending`` and a
-# fused launch) or, like any other call into the library, finds it run first -- ``call`` flushes
+# once: its caller parks it here.  The next operation either takes it over (``take_pending_if`` and
+# a fused launch) or, like any other call into the library, finds it run first -- ``call`` flushes
 # before it does anything else, so a deferred operation never outlives the next library call and
 # nothing can read or overwrite its operands in between.
+#
+# The slot is shared by all threads (a buffer that thread A's parked operation will fill may be
+# read by thread B, whose first use of it must find the operation run), so every access goes
+# through one re-entrant lock: parking, the test-and-take of a fusing successor and the flush are
+# each atomic, and a flush started by one thread is finished before another thread's call proceeds.
 _pending = None
+_lock = threading.RLock()
 
 
 def defer(op):
     """Park ``op`` (an object with ``run()``); whatever was parked before runs now."""
     global _pending
-    flush()
-    _pending = op
+    with _lock:
+        flush()
+        _pending = op
 
 
 def pending():
@@ -140,14 +155,38 @@ def pending():
 
 def take_pending():
     global _pending
-    op, _pending = _pending, None
+    with _lock:
+        op, _pending = _pending, None
+    return op
+
+
+def take_pending_if(wanted):
+    """The parked operation, removed from the slot, if ``wanted(op)`` holds for it -- test and take
+    in one step, so that no other thread can run or steal it in between; otherwise None (and the
+    operation stays parked)."""
+    global _pending
+    with _lock:
+        op = _pending
+        if op is None or not wanted(op):
+            return None
+        _pending = None
     return op
 
 
 def flush():
-    op = take_pending()
-    if op is not None:
-        op.run()
+    """Run the parked operation, if any.  Should it fail, the arrays it was to fill are marked:
+    any later use of them raises the same error instead of reading memory nobody wrote."""
+    with _lock:
+        op = take_pending()
+        if op is None:
+            return
+        try:
+            op.run()
+        except Exception as exc:
+            poison = getattr(op, 'poison', None)
+            if poison is not None:
+                poison(exc)
+            raise
 
 
 def call(name, *args):

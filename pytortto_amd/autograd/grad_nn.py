@@ -167,11 +167,10 @@ class BatchNorm(Function):
         gd0, = grad_outputs
         xd0, xd1 = ctx.saved_tensors
         p = ctx.params
-        parked = _hip.pending()
-        if parked.__class__ is ops.DeferredReluBackward and parked.out._buf is gd0._buf:
+        parked = _hip.take_pending_if(lambda op: op.__class__ is ops.DeferredReluBackward and op.out._buf is gd0._buf)
+        if parked is not None:
             # the gradient comes straight from a ReLU whose mask has not been applied yet: apply it
             # while reading dy (grad_nn.py:67 folded into :977-988)
-            _hip.take_pending()
             return ops.bn_relu_bwd(xd0, parked.dy, parked.y, xd1, p['mean'], p['var'], p['sd'],
                                    need=ctx.needs_input_grad)
         grad0, grad1, grad2 = ops.bn_bwd(xd0, gd0, xd1, p['mean'], p['var'], p['sd'], need=ctx.needs_input_grad)
@@ -184,25 +183,26 @@ class Relu(Function):
         xt0, = inputs
         xd0 = xt0.data
         inplace = params['inplace']
-        parked = _hip.pending()
-        if parked.__class__ is ops.DeferredBatchNorm and parked.y._buf is xd0._buf:
-            # the input is a BatchNorm output that has not been launched yet: one kernel writes
-            # maximum(bn(x), 0) directly (grad_nn.py:942-959 and :56 in one pass)
+        # only a device input can be the output of a parked device operation (a host array has no buffer)
+        parked = None
+        if xd0.__class__ is hiparray:
+            parked = _hip.take_pending_if(lambda op: (op.__class__ is ops.DeferredBatchNorm and op.y._buf is xd0._buf)
+                                          or (op.__class__ is ops.DeferredAdd and op.out._buf is xd0._buf))
+        if parked is not None:
+            # the input is a BatchNorm output, or a residual sum, that has not been launched yet: one
+            # kernel writes maximum(bn(x), 0) (grad_nn.py:942-959 and :56 in one pass) or maximum(a + b, 0)
             if inplace:
-                inplace_precheck(xt0)
-                _hip.take_pending().run_with_relu()
+                try:
+                    inplace_precheck(xt0)
+                except RuntimeError:
+                    parked.run()
+                    raise
+                parked.run_with_relu()
                 yt0 = inplace_update(xt0, ctx)
             else:
-                yt0 = build_links(_hip.take_pending().run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
-            ctx.params['after_batch_norm'] = True
-        elif parked.__class__ is ops.DeferredAdd and parked.out._buf is xd0._buf:
-            # the input is a residual sum that has not been launched yet: maximum(a + b, 0) in one pass
-            if inplace:
-                inplace_precheck(xt0)
-                _hip.take_pending().run_with_relu()
-                yt0 = inplace_update(xt0, ctx)
-            else:
-                yt0 = build_links(_hip.take_pending().run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
+                yt0 = build_links(parked.run_with_relu(hiparray.empty(xd0.shape)), grad_fn=ctx)
+            if parked.__class__ is ops.DeferredBatchNorm:
+                ctx.params['after_batch_norm'] = True
         elif xd0.__class__ is hiparray:
             if inplace:
                 inplace_precheck(xt0)
@@ -292,19 +292,14 @@ def _reference_pos(tap, kw):
 class MaxPool2DWithIndices(Function):
     @staticmethod
     def forward(ctx, *inputs, **params):
-        xt0, = inputs
-        xd0 = xt0.data
-        kernel_size = params['kernel_size']
-        stride = params['stride']
-        padding = params['padding']
-        dilation = params['dilation']
-        ceil_mode = params['ceil_mode']
-        return_indices = params['return_indices']
-        if padding[0] * 2 > kernel_size[0] or padding[1] * 2 > kernel_size[1]:
+        (xt0,), xd0 = inputs, inputs[0].data
+        kernel_size, stride, padding, dilation, ceil_mode, return_indices = (
+            params[name] for name in ('kernel_size', 'stride', 'padding', 'dilation', 'ceil_mode', 'return_indices'))
+        (kh, kw), (pad_h, pad_w) = kernel_size, padding
+        if 2 * pad_h > kh or 2 * pad_w > kw:        # the reference's two checks and messages (grad_nn.py:835-845)
             raise RuntimeError(f'pad should be smaller than or equal to half of kernel size, '
-                               f'but got padW = {padding[1]}, padH = {padding[0]}, kW = {kernel_size[1]}, '
-                               f'kH = {kernel_size[0]}')
-        if xd0.ndim != 3 and xd0.ndim != 4:
+                               f'but got padW = {pad_w}, padH = {pad_h}, kW = {kw}, kH = {kh}')
+        if xd0.ndim not in (3, 4):
             raise RuntimeError('non-empty 3D or 4D (batch mode) tensor expected for input')
         _device_only('max_pool2d', xd0)
         out_hw = tuple(pool_output_size(xd0.shape[-2 + a], kernel_size[a], stride[a], padding[a], dilation[a],

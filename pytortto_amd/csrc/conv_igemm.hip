@@ -30,6 +30,7 @@
 // Optional reduced-precision variant (tt_set_conv_math(TT_CONV_MATH_BF16)): the same kernels with
 // the operands rounded to bfloat16 after the LDS read and contracted by v_mfma_f32_32x32x16_bf16,
 // float32 accumulation, float32 tensors in memory.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -110,6 +111,7 @@ struct Igemm {
   floatx4* skPartial;        // [skBlocks][acc float4s per thread][256] partial accumulators, one slot per block
   unsigned* skFlags;         // [block] = skEpoch once the block's partial is in memory
   unsigned skEpoch;          // differs from launch to launch, so the flags never need clearing
+  unsigned* skError;         // one word in pinned host memory: set when a wait for a flag ran out
 };
 
 // ---- preparation kernels (tiny) --------------------------------------------------------------
@@ -254,10 +256,11 @@ __device__ __forceinline__ void wait_loads() {
 // costs.  Ordering is by completion: the writer waits for its stores (vmcnt) before the flag goes
 // up, the reader issues its loads after it has seen the flag.
 constexpr int kSystemScope = 1 | 16;   // sc0, sc1
-// stream-K flags: one word per block, the last word of the array reports a wait that ran out
-// (about four seconds of polling: a block that was never scheduled, i.e. a grid that does not fit
-// the device at two blocks per CU next to foreign work)
-constexpr int kSkFlagWords = 4096, kSkErrorWord = kSkFlagWords - 1, kSkSpinLimit = 1 << 22;
+// stream-K flags: one word per block.  A wait that runs out (about four seconds of polling: a block
+// that was never scheduled, i.e. a grid that does not fit the device at two blocks per CU next to
+// foreign work) is reported through a word in pinned host memory, which the host reads after its
+// next stream synchronisation without any device operation.
+constexpr int kSkFlagWords = 4096, kSkSpinLimit = 1 << 22;
 __device__ __forceinline__ void store_coherent(__amdgpu_buffer_rsrc_t rsrc, int byte_off, floatx4 v) {
   typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
   __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, v), rsrc, byte_off, 0, kSystemScope);
@@ -828,11 +831,15 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
         const long long t0 = (long long)t_first * chunks;
         const int b_first = (int)(((t0 + 1) * p.skBlocks - 1) / p.skIters);
         if (tid == 0) {
-          for (int j = b_first; j < b; ++j) {
+          bool lost = false;
+          for (int j = b_first; j < b && !lost; ++j) {
             int spins = 0;
             while (__hip_atomic_load(&p.skFlags[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != p.skEpoch) {
-              if (++spins >= kSkSpinLimit) {   // never hang: give up, flag the launch as failed
-                __hip_atomic_store(&p.skFlags[kSkErrorWord], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+              if (++spins >= kSkSpinLimit) {
+                // never hang: give up, report the launch as failed, and do not wait for the
+                // remaining predecessors either (one spin budget per block, not one per predecessor)
+                __hip_atomic_store(p.skError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                lost = true;
                 break;
               }
               __builtin_amdgcn_s_sleep(4);
@@ -954,9 +961,39 @@ TileChoice choose_tile(int I, int M, int groups, int chunks, bool allow_stream_k
 // bytes of stream-K partial accumulators for the largest tile: one slot per block
 size_t sk_workspace_bytes() { return (size_t)sk_launch_blocks() * 128 * 128 * sizeof(float); }
 
+// The stream-K wait is safe only while every block of the persistent grid is resident at once
+// (sk_launch_blocks() = 2 per CU, 3 for the bf16 kernels).  What the device can hold of one
+// instantiation is asked once (registers and LDS of the compiled kernel decide it); an
+// instantiation that cannot hold that many is launched data-parallel instead, one tile per block:
+// a register-count regression then costs speed, never a stalled launch.
+template <int WM, int WN, int MT, int NT, int MODE, bool AT, bool BFK>
+int sk_resident_blocks_per_cu() {
+  static int cached = -1;
+  if (cached < 0) {
+    int n = 0;
+    hipError_t e;
+    if constexpr (BFK) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_bf16<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
+    else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_f32<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      n = 0;
+    }
+    cached = n;
+  }
+  return cached;
+}
+int g_sk_forced_occupancy = -1;   // >= 0: pretend every instantiation holds this many blocks per CU (tests of the fallback)
+
+// Returns whether the persistent (stream-K) grid was launched.
 template <int WM, int WN, int MT, int NT, int MODE, bool AT>
-void launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+bool launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
+  if (sk_blocks > 0) {
+    int held = bf ? sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, true>()
+                  : sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, false>();
+    if (g_sk_forced_occupancy >= 0) held = g_sk_forced_occupancy;
+    if ((long long)held * cus() < sk_blocks) sk_blocks = 0;   // the data-parallel launch ignores the stream-K fields
+  }
   if (sk_blocks > 0) {
     if (bf) igemm_bf16<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     else igemm_f32<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
@@ -965,16 +1002,38 @@ void launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   } else {
     igemm_f32<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
+  return sk_blocks > 0;
+}
+// smallest number of resident blocks per CU over every stream-K instantiation of one tile shape
+template <int WM, int WN, int MT, int NT, bool BFK>
+int sk_min_resident() {
+  const int all[] = {sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeGemm, true, BFK>(),
+                     sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeGemm, false, BFK>(),
+                     sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeTapMask, true, BFK>(),
+                     sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeTapMask, false, BFK>(),
+                     sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeTapMask64, false, BFK>(),
+                     sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeCompare, false, BFK>()};
+  int lo = all[0];
+  for (int v : all) lo = v < lo ? v : lo;
+  return lo;
+}
+template <bool BFK>
+int sk_min_resident_all() {
+  const int all[] = {sk_min_resident<2, 2, 2, 2, BFK>(), sk_min_resident<1, 4, 2, 2, BFK>(),
+                     sk_min_resident<1, 4, 1, 2, BFK>(), sk_min_resident<2, 2, 1, 1, BFK>()};
+  int lo = all[0];
+  for (int v : all) lo = v < lo ? v : lo;
+  return lo;
 }
 template <int WM, int WN, int MT, int NT>
-void launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
+bool launch_config(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
   const bool at = p.wTransStride > 0;
-  if (p.mode == kModeGemm && at) launch_mode<WM, WN, MT, NT, kModeGemm, true>(p, groups, sk_blocks, st);
-  else if (p.mode == kModeGemm) launch_mode<WM, WN, MT, NT, kModeGemm, false>(p, groups, sk_blocks, st);
-  else if (p.mode == kModeTapMask && at) launch_mode<WM, WN, MT, NT, kModeTapMask, true>(p, groups, sk_blocks, st);
-  else if (p.mode == kModeTapMask) launch_mode<WM, WN, MT, NT, kModeTapMask, false>(p, groups, sk_blocks, st);
-  else if (p.mode == kModeTapMask64) launch_mode<WM, WN, MT, NT, kModeTapMask64, false>(p, groups, sk_blocks, st);
-  else launch_mode<WM, WN, MT, NT, kModeCompare, false>(p, groups, sk_blocks, st);
+  if (p.mode == kModeGemm && at) return launch_mode<WM, WN, MT, NT, kModeGemm, true>(p, groups, sk_blocks, st);
+  if (p.mode == kModeGemm) return launch_mode<WM, WN, MT, NT, kModeGemm, false>(p, groups, sk_blocks, st);
+  if (p.mode == kModeTapMask && at) return launch_mode<WM, WN, MT, NT, kModeTapMask, true>(p, groups, sk_blocks, st);
+  if (p.mode == kModeTapMask) return launch_mode<WM, WN, MT, NT, kModeTapMask, false>(p, groups, sk_blocks, st);
+  if (p.mode == kModeTapMask64) return launch_mode<WM, WN, MT, NT, kModeTapMask64, false>(p, groups, sk_blocks, st);
+  return launch_mode<WM, WN, MT, NT, kModeCompare, false>(p, groups, sk_blocks, st);
 }
 
 // Picks how the kernel addresses the gathered operand (see Igemm::mode) and completes the table
@@ -1012,6 +1071,26 @@ void choose_mode(Igemm& p, KTabArgs& ka, bool gemm_geometry, int N, int U, int V
 // so the words never need clearing again.
 unsigned g_sk_epoch = 0;
 unsigned* g_sk_flags = nullptr;
+// The word a block sets when its wait ran out: pinned host memory mapped into the device's address
+// space, so the host reads it directly once the stream has drained.
+volatile unsigned* g_sk_error_host = nullptr;
+unsigned* g_sk_error_dev = nullptr;
+int sk_error_word(unsigned** out) {
+  if (g_sk_error_host == nullptr) {
+    void* host = nullptr;
+    TT_HIP(hipHostMalloc(&host, sizeof(unsigned), hipHostMallocMapped));
+    *(volatile unsigned*)host = 0u;
+    void* dev = nullptr;
+    if (hipError_t e = hipHostGetDevicePointer(&dev, host, 0); e != hipSuccess) {
+      (void)hipHostFree(host);
+      return tt::fail_hip(e, "hipHostGetDevicePointer", __FILE__, __LINE__);
+    }
+    g_sk_error_host = (volatile unsigned*)host;
+    g_sk_error_dev = (unsigned*)dev;
+  }
+  *out = g_sk_error_dev;
+  return 0;
+}
 int sk_flags(unsigned** out) {
   if (g_sk_flags == nullptr) {
     const size_t bytes = sizeof(unsigned) * kSkFlagWords;
@@ -1021,6 +1100,14 @@ int sk_flags(unsigned** out) {
   *out = g_sk_flags;
   return 0;
 }
+
+// Sets the error word from the device, exactly as a block whose wait ran out does.
+__global__ void sk_raise_error(unsigned* word) {
+  __hip_atomic_store(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// What the last single launch looked like (instrumentation: tests pick the images to compare from it).
+int g_last_launch[8] = {};
 
 int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_partial) {
   tt::ProfScope prof(prof_id);
@@ -1039,20 +1126,29 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
       if (share < rem) share = rem;
       p.skBlocks = (int)(share < t.sk_blocks ? share : t.sk_blocks);
       p.skPartial = sk_partial;
-      if (sk_flags(&p.skFlags)) return -1;
+      if (sk_flags(&p.skFlags) || sk_error_word(&p.skError)) return -1;
       if (++g_sk_epoch == 0) ++g_sk_epoch;
       p.skEpoch = g_sk_epoch;
     }
   }
+  const int plan[8] = {t.bm, t.bn, p.tiles, p.tilesI, t.sk_blocks, t.sk_blocks > 0 ? p.skDpTiles : p.tiles,
+                       t.sk_blocks > 0 ? p.skBlocks : 0, p.mode};
+  std::copy(plan, plan + 8, g_last_launch);
   hipStream_t st = tt::stream();
+  bool persistent;
   if (t.bm == 128 && t.bn == 128)
-    launch_config<2, 2, 2, 2>(p, groups, t.sk_blocks, st);
+    persistent = launch_config<2, 2, 2, 2>(p, groups, t.sk_blocks, st);
   else if (t.bm == 64 && t.bn == 256)
-    launch_config<1, 4, 2, 2>(p, groups, t.sk_blocks, st);
+    persistent = launch_config<1, 4, 2, 2>(p, groups, t.sk_blocks, st);
   else if (t.bm == 32 && t.bn == 256)
-    launch_config<1, 4, 1, 2>(p, groups, t.sk_blocks, st);
+    persistent = launch_config<1, 4, 1, 2>(p, groups, t.sk_blocks, st);
   else
-    launch_config<2, 2, 1, 1>(p, groups, t.sk_blocks, st);
+    persistent = launch_config<2, 2, 1, 1>(p, groups, t.sk_blocks, st);
+  if (!persistent) {   // also when the device could not hold the persistent grid: one tile per block
+    g_last_launch[4] = 0;
+    g_last_launch[5] = p.tiles;
+    g_last_launch[6] = 0;
+  }
   TT_LAUNCH_CHECK();
   return 0;
 }
@@ -1313,11 +1409,8 @@ int conv_release_tables() { return release_tables(); }
 // After a stream sync: has a stream-K block given up waiting for another block's partial sums since
 // the last check?  The convolution results since then are invalid in that case.
 int conv_check_async_error() {
-  if (g_sk_flags == nullptr) return 0;
-  unsigned word = 0;
-  TT_HIP(hipMemcpy(&word, g_sk_flags + kSkErrorWord, sizeof(word), hipMemcpyDeviceToHost));
-  if (word == 0) return 0;
-  TT_HIP(hipMemset(g_sk_flags + kSkErrorWord, 0, sizeof(word)));
+  if (g_sk_error_host == nullptr || *g_sk_error_host == 0u) return 0;
+  *g_sk_error_host = 0u;   // the stream has drained: no kernel that could set it is running
   return tt::fail(-1, "a convolution launch timed out waiting for another block's partial sums (the device could not "
                       "hold its grid of two blocks per compute unit); convolution results since the last "
                       "synchronisation are invalid");
@@ -1328,8 +1421,48 @@ extern "C" {
 
 int tt_set_conv_dense_cell_min_tiles(int tiles) {
   TT_API_LOCK();
-  TT_REQUIRE(tiles >= 0 && tiles <= (1 << 20), "tt_set_conv_dense_cell_min_tiles: %d is out of range (0..2^20)", tiles);
-  g_dense_cell_min_tiles = tiles;
+  TT_REQUIRE(tiles >= -1 && tiles <= (1 << 20), "tt_set_conv_dense_cell_min_tiles: %d is out of range (-1..2^20)", tiles);
+  g_dense_cell_min_tiles = tiles;   // -1: back to the default, 1.5 tiles per compute unit
+  return 0;
+}
+
+// Instrumentation (tests): resident blocks per compute unit of the stream-K kernels, the smallest
+// over every instantiation, float32 (bf16 == 0) or bf16 ones.  The launches need 2 resp. 3.
+int tt_conv2d_stream_k_blocks_per_cu(int bf16, int* blocks) {
+  TT_REQUIRE_INIT();
+  TT_REQUIRE(blocks != nullptr, "tt_conv2d_stream_k_blocks_per_cu: null result pointer");
+  *blocks = bf16 ? sk_min_resident_all<true>() : sk_min_resident_all<false>();
+  return 0;
+}
+
+// Instrumentation (tests): the plan of the last single matrix-product launch of a forward or input
+// gradient call: {tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent grid
+// (0: one tile per block), tiles computed whole (the rest share their reduction between blocks),
+// blocks sharing them, addressing mode}.  Pixel tile t starts at pixel (t / row tiles) * tile columns.
+int tt_conv2d_last_launch(int* plan8) {
+  TT_API_LOCK();
+  TT_REQUIRE(plan8 != nullptr, "tt_conv2d_last_launch: null result pointer");
+  std::copy(g_last_launch, g_last_launch + 8, plan8);
+  return 0;
+}
+
+// Instrumentation (tests): pretend that every stream-K instantiation holds `blocks` blocks per
+// compute unit (-1: ask the device again), so that the data-parallel fallback can be exercised.
+int tt_conv2d_stream_k_force_occupancy(int blocks) {
+  TT_API_LOCK();
+  TT_REQUIRE(blocks >= -1 && blocks <= 64, "tt_conv2d_stream_k_force_occupancy: %d is out of range (-1..64)", blocks);
+  g_sk_forced_occupancy = blocks;
+  return 0;
+}
+
+// Instrumentation (tests): a one-thread kernel sets the word that a stream-K block sets when its
+// wait for another block runs out.  The next tt_sync() / tt_memcpy_d2h() must report it, once.
+int tt_conv2d_selftest_raise_async_error(void) {
+  TT_REQUIRE_INIT();
+  unsigned* word = nullptr;
+  if (sk_error_word(&word)) return -1;
+  sk_raise_error<<<1, 1, 0, tt::stream()>>>(word);
+  TT_LAUNCH_CHECK();
   return 0;
 }
 
@@ -1694,11 +1827,17 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
 // The kernels index with 32-bit element offsets.  Forward and input gradient are independent per
 // image, so a batch whose tensors have 2^31 elements or more runs as several calls over runs of
 // images that stay below that (one image and the weights must fit on their own).
+// Every run but the first starts `per` images into the tensors, and the kernels need 16-byte
+// aligned pointers: `per` is rounded down until both tensors' runs are whole float4s long (one of
+// four consecutive counts always is).  0: not even one image per run can be kept aligned.
 static int images_per_call(int N, long long image_a, long long image_b) {
   const long long image = image_a > image_b ? image_a : image_b;
   if (N <= 0 || image <= 0 || (long long)N * image < 2147483647LL) return N;
-  const long long per = 2147483646LL / image;
-  return (int)(per < 1 ? 1 : per);
+  long long per = 2147483646LL / image;
+  if (per < 1) per = 1;
+  for (long long cand = per; cand >= 1 && cand > per - 4; --cand)
+    if ((cand * image_a) % 4 == 0 && (cand * image_b) % 4 == 0) return (int)cand;
+  return 0;
 }
 static long long out_size(long long in, int k, int s, int p, int d) { return (in + 2LL * p - (long long)d * (k - 1) - 1) / s + 1; }
 
@@ -1707,6 +1846,8 @@ int tt_conv2d_fwd_f32(const float* x, const float* w, const float* bias, float* 
   const long long xi = (long long)C * H * W;
   const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
   const int per = images_per_call(N, xi, yi);
+  TT_REQUIRE(per > 0, "tt_conv2d_fwd_f32: a batch of 2^31 elements or more is cut into runs of images, and images of "
+                      "%lld and %lld elements leave no run 16-byte aligned", xi, yi);
   if (per >= N) return conv2d_fwd(x, w, bias, y, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr);
   for (int n0 = 0; n0 < N; n0 += per) {
     const int n = N - n0 < per ? N - n0 : per;
@@ -1722,6 +1863,8 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
                         int Q) {
   const long long xi = (long long)C * Hx * Wx, yi = (long long)K * P * Q;
   const int per = images_per_call(N, xi, yi);
+  TT_REQUIRE(per > 0, "tt_conv2d_dgrad_f32: a batch of 2^31 elements or more is cut into runs of images, and images of "
+                      "%lld and %lld elements leave no run 16-byte aligned", xi, yi);
   if (per >= N) return conv2d_dgrad(dy, w, bias, dx, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q, nullptr);
   for (int n0 = 0; n0 < N; n0 += per) {
     const int n = N - n0 < per ? N - n0 : per;
@@ -1732,19 +1875,27 @@ int tt_conv2d_dgrad_f32(const float* dy, const float* w, const float* bias, floa
   return 0;
 }
 
+// Instrumentation (tests, host-only): images per run for a batch of N images of `image_a` and
+// `image_b` elements (input and output of a forward or input-gradient call); 0 = no aligned run.
+int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* per) {
+  TT_REQUIRE(per != nullptr, "tt_conv2d_images_per_run: null result pointer");
+  *per = images_per_call(N, image_a, image_b);
+  return 0;
+}
+
 // Host-only: builds every index table the corresponding call would use for this geometry and checks
 // each entry's reach against the tensors, as the calls themselves do once per new geometry.
 int tt_conv2d_check_tables_fwd_f32(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
                                    int dh, int dw, int groups) {
   const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
-  N = images_per_call(N, (long long)C * H * W, yi);
+  N = std::max(1, images_per_call(N, (long long)C * H * W, yi));
   return conv2d_fwd(nullptr, nullptr, nullptr, nullptr, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups, nullptr,
                     true);
 }
 
 int tt_conv2d_check_tables_dgrad_f32(int N, int C, int Hx, int Wx, int K, int R, int S, int sh, int sw, int ph, int pw,
                                      int dh, int dw, int groups, int P, int Q) {
-  N = images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q);
+  N = std::max(1, images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q));
   return conv2d_dgrad(nullptr, nullptr, nullptr, nullptr, N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups, P, Q,
                       nullptr, true);
 }
@@ -1784,7 +1935,7 @@ int tt_workspace_size_conv2d_fwd_f32(size_t* bytes, int N, int C, int H, int W, 
   TT_REQUIRE(bytes, "tt_workspace_size_conv2d_fwd_f32: null result pointer");
   const float* in = reinterpret_cast<const float*>(uintptr_t(256));
   const long long yi = sh > 0 && sw > 0 ? (long long)K * out_size(H, R, sh, ph, dh) * out_size(W, S, sw, pw, dw) : 0;
-  N = images_per_call(N, (long long)C * H * W, yi);   // the largest of the calls a long batch is cut into
+  N = std::max(1, images_per_call(N, (long long)C * H * W, yi));   // the largest of the calls a long batch is cut into
   return conv2d_fwd(in, in, nullptr, const_cast<float*>(in), N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups,
                     bytes);
 }
@@ -1793,7 +1944,7 @@ int tt_workspace_size_conv2d_dgrad_f32(size_t* bytes, int N, int C, int Hx, int 
                                        int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q) {
   TT_REQUIRE(bytes, "tt_workspace_size_conv2d_dgrad_f32: null result pointer");
   const float* in = reinterpret_cast<const float*>(uintptr_t(256));
-  N = images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q);
+  N = std::max(1, images_per_call(N, (long long)C * Hx * Wx, (long long)K * P * Q));
   return conv2d_dgrad(in, in, nullptr, const_cast<float*>(in), N, C, Hx, Wx, K, R, S, sh, sw, ph, pw, dh, dw, groups,
                       P, Q, bytes);
 }

@@ -55,8 +55,6 @@ struct Wgrad {
   size_t outStrideSplit;      // G*Kg*J
   int R, S;                   // buffer path: taps, one bit each in the per-chunk mask
   int xBias;                  // buffer path: ph*W + pw, keeps lane offsets non-negative
-  tt::FastDiv divDh, divDw;   // buffer path: division by the dilation
-  uint32_t rowOnes;           // buffer path: bit r*S set for every tap row r
   // buffer path: per output pixel m {image n, 4*(p*Q + q), 4*(ih*W + iw + xBias), tap mask};
   // entries from M to chunks*32 hold {N-1, bit 31, 0, all ones}.  Built once per geometry.
   const int4* pixtab;
@@ -66,67 +64,6 @@ struct Wgrad {
 constexpr int kSrdFlags = 0x00020000;     // raw buffer, 32-bit data format
 constexpr int kSrdRecords = 0x7fffffff;   // offsets with bit 31 set are out of range and read 0
 __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
-
-// Taps t = 0..n-1 sit at pos + t*step; those with 0 <= pos + t*step < lim form a range [lo, hi].
-// Returns the bits [lo*unit, (hi+1)*unit) (n*unit <= 31), without a loop.
-__device__ __forceinline__ uint32_t tap_range_bits(int pos, int lim, int n, int unit, const tt::FastDiv& step) {
-  int lo = pos >= 0 ? 0 : (int)tt::fd_div((uint32_t)(-pos + (int)step.d - 1), step);
-  const int room = lim - 1 - pos;
-  const int hi = room < 0 ? -1 : min(n - 1, (int)tt::fd_div((uint32_t)room, step));
-  lo = min(lo, n);
-  const uint32_t upto = (1u << ((hi + 1) * unit)) - 1u, below = (1u << (lo * unit)) - 1u;
-  return lo > hi ? 0u : upto & ~below;
-}
-
-// The same for masks of up to 63 bits (n*unit <= 63).
-__device__ __forceinline__ uint64_t tap_range_bits64(int pos, int lim, int n, int unit, const tt::FastDiv& step) {
-  int lo = pos >= 0 ? 0 : (int)tt::fd_div((uint32_t)(-pos + (int)step.d - 1), step);
-  const int room = lim - 1 - pos;
-  const int hi = room < 0 ? -1 : min(n - 1, (int)tt::fd_div((uint32_t)room, step));
-  lo = min(lo, n);
-  const uint64_t upto = (1ull << ((hi + 1) * unit)) - 1ull, below = (1ull << (lo * unit)) - 1ull;
-  return lo > hi ? 0ull : upto & ~below;
-}
-
-// Pixel table of the buffer path: what the main loop would otherwise recompute for every chunk
-// in every block (two divisions, the tap ranges) depends only on the geometry.
-// `hi` (kernels of 32 .. 63 taps only): receives the upper half of each 64-bit mask.
-__global__ void wgrad_build_pixtab(int4* __restrict__ tab, int* __restrict__ hi, Wgrad p, int entries, int N) {
-  const int m = blockIdx.x * blockDim.x + threadIdx.x;
-  if (m >= entries) return;
-  int4 e = make_int4(N - 1, (int)0x80000000u, 0, -1);
-  if (hi != nullptr) {
-    uint64_t outside = ~0ull;
-    if (m < p.M) {
-      const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
-      const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
-      const uint32_t pp = tt::fd_div(pq, p.divQ);
-      const uint32_t qq = pq - pp * p.divQ.d;
-      const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
-      uint64_t row_ones = 0;
-      for (int r = 0; r < p.R; ++r) row_ones |= 1ull << (r * p.S);
-      const uint64_t cols = tap_range_bits64(iw, p.W, p.S, 1, p.divDw);
-      const uint64_t rows = tap_range_bits64(ih, p.H, p.R, p.S, p.divDh) & row_ones;
-      outside = ~(cols * rows);   // bit 63 stays set: R*S <= 63
-      e = make_int4((int)n, 4 * (int)pq, 4 * (ih * p.W + iw + p.xBias), (int)(uint32_t)outside);
-    }
-    tab[m] = e;
-    hi[m] = (int)(uint32_t)(outside >> 32);
-    return;
-  }
-  if (m < p.M) {
-    const uint32_t n = tt::fd_div((uint32_t)m, p.divPQ);
-    const uint32_t pq = (uint32_t)m - n * p.divPQ.d;
-    const uint32_t pp = tt::fd_div(pq, p.divQ);
-    const uint32_t qq = pq - pp * p.divQ.d;
-    const int ih = (int)pp * p.sh - p.ph, iw = (int)qq * p.sw - p.pw;
-    // valid tap columns, replicated into every valid tap row (fields of S bits: no carries)
-    const uint32_t cols = tap_range_bits(iw, p.W, p.S, 1, p.divDw);
-    const uint32_t rows = tap_range_bits(ih, p.H, p.R, p.S, p.divDh) & p.rowOnes;
-    e = make_int4((int)n, 4 * (int)pq, 4 * (ih * p.W + iw + p.xBias), (int)~(cols * rows));   // bit 31 stays set: R*S <= 31
-  }
-  tab[m] = e;
-}
 
 // Two blocks per CU is all the LDS tiles allow: tell the compiler not to squeeze registers (and
 // spill) for a third wave per SIMD.
@@ -525,20 +462,152 @@ __global__ __launch_bounds__(kThreads) void wgrad_reduce(const float* __restrict
 
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+// ---- pixel table -------------------------------------------------------------------------------------
+// What the main loop would otherwise recompute for every chunk in every block (two divisions, the
+// tap ranges) depends only on the geometry: per output pixel m = (n, p, q)
+//   {image n, byte offset 4*(p*Q + q) of the pixel in a dy plane,
+//    byte offset 4*(ih*W + iw + xBias) of the window's first tap in an x plane, tap mask}
+// (bit t of the mask set: tap t = r*S + s lies outside the image for this pixel; kernels of
+// 32 .. 63 taps keep bits 32 .. 63 in a second array).  Entries from M to chunks*32 hold
+// {N-1, bit 31, 0, all ones}: a pixel past the end reads zeros everywhere.
+// The table is built on the host, checked there against the two tensors it indexes, uploaded once
+// into a device buffer of its own and kept per geometry: no kernel writes it.
+struct PixGeom {
+  int N, C, K, groups, P, Q, H, W, R, S, sh, sw, ph, pw, dh, dw, chunks;
+};
+struct HostPixTab {
+  std::vector<int4> tab;
+  std::vector<int> hi;   // empty unless the kernel has 32 .. 63 taps
+};
+
+// Floor and ceiling of a / b for b > 0 and any a.
+long long floor_div(long long a, long long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+long long ceil_div_s(long long a, long long b) { return -floor_div(-a, b); }
+
+// Taps t = 0 .. n-1 at pos + t*step: bits [lo*unit, (hi+1)*unit) for the range [lo, hi] of taps that
+// fall inside [0, lim) (closed form, as the lanes used to compute it).
+uint64_t tap_range_bits_host(int pos, int lim, int n, int unit, int step) {
+  long long lo = std::max<long long>(0, ceil_div_s(-(long long)pos, step));
+  long long hi = std::min<long long>(n - 1, floor_div((long long)lim - 1 - pos, step));
+  if (lo > hi) return 0;
+  const uint64_t upto = (hi + 1) * unit >= 64 ? ~0ull : (1ull << ((hi + 1) * unit)) - 1ull;
+  const uint64_t below = (1ull << (lo * unit)) - 1ull;
+  return upto & ~below;
+}
+
+void build_pixtab(const PixGeom& g, bool wide, HostPixTab* out) {
+  const int PQ = g.P * g.Q, M = g.N * PQ, entries = g.chunks * kBK;
+  const int xBias = g.ph * g.W + g.pw;
+  out->tab.assign((size_t)entries, make_int4(g.N - 1, (int)0x80000000u, 0, -1));
+  out->hi.assign(wide ? (size_t)entries : 0, -1);
+  uint64_t row_ones = 0;
+  for (int r = 0; r < g.R; ++r) row_ones |= 1ull << (r * g.S);
+  // the part that depends on (p, q) only, once; then one entry per image
+  std::vector<int4> plane((size_t)PQ);
+  std::vector<int> plane_hi(wide ? (size_t)PQ : 0);
+  for (int pq = 0; pq < PQ; ++pq) {
+    const int pp = pq / g.Q, qq = pq % g.Q;
+    const int ih = pp * g.sh - g.ph, iw = qq * g.sw - g.pw;
+    // valid tap columns, replicated into every valid tap row (fields of S bits: no carries)
+    const uint64_t cols = tap_range_bits_host(iw, g.W, g.S, 1, g.dw);
+    const uint64_t rows = tap_range_bits_host(ih, g.H, g.R, g.S, g.dh) & row_ones;
+    const uint64_t outside = ~(cols * rows);   // the top bit stays set: R*S <= 31 (63)
+    plane[(size_t)pq] = make_int4(0, 4 * pq, 4 * (ih * g.W + iw + xBias), (int)(uint32_t)outside);
+    if (wide) plane_hi[(size_t)pq] = (int)(uint32_t)(outside >> 32);
+  }
+  for (int m = 0; m < M; ++m) {
+    int4 e = plane[(size_t)(m % PQ)];
+    e.x = m / PQ;
+    out->tab[(size_t)m] = e;
+    if (wide) out->hi[(size_t)m] = plane_hi[(size_t)(m % PQ)];
+  }
+}
+
+// What the kernel will do with every entry, replayed on the host: the dy element a lane fetches for
+// the entry's pixel must be pixel (n, p, q) of the row's plane and lie inside dy; for every tap the
+// mask lets through, the x element must be (n, c, p*sh - ph + r*dh, q*sw - pw + s*dw), inside its
+// image -- and every tap the mask blocks must really fall outside, or a product would be lost
+// silently; 32-bit byte offsets relative to the first image of a chunk (at most 33 images back)
+// must stay in [0, 2^31); entries past the end must read zeros.
+int check_pixtab(const char* fn, const PixGeom& g, bool wide, const HostPixTab& t) {
+  const int PQ = g.P * g.Q, M = g.N * PQ, entries = g.chunks * kBK;
+  const int taps = g.R * g.S, top = wide ? 63 : 31;
+  const int Cg = g.C / g.groups, Kg = g.K / g.groups;
+  const long long xImg = (long long)g.C * g.H * g.W, dyImg = (long long)g.K * PQ;
+  const long long xBias = (long long)g.ph * g.W + g.pw;
+  TT_REQUIRE((int)t.tab.size() == entries && (wide ? (int)t.hi.size() == entries : t.hi.empty()) && entries >= M &&
+                 taps <= top,
+             "%s: pixel table of %zu entries for %d pixels in %d chunks, %d taps", fn, t.tab.size(), M, g.chunks, taps);
+  auto mask_of = [&](int m) {
+    return wide ? ((uint64_t)(uint32_t)t.hi[(size_t)m] << 32) | (uint32_t)t.tab[(size_t)m].w
+                : (uint64_t)(uint32_t)t.tab[(size_t)m].w;
+  };
+  // the (p, q)-dependent fields, pixel by pixel of the first image
+  for (int pq = 0; pq < std::min(PQ, M); ++pq) {
+    const int4 e = t.tab[(size_t)pq];
+    const int pp = pq / g.Q, qq = pq % g.Q;
+    TT_REQUIRE(e.y == 4 * pq, "%s: pixel table entry %d: dy byte offset %d for pixel (%d, %d)", fn, pq, e.y, pp, qq);
+    const uint64_t outside = mask_of(pq);
+    TT_REQUIRE((outside >> top) & 1, "%s: pixel table entry %d: the padding tap %d is not blocked", fn, pq, top);
+    const long long first = e.z / 4 - xBias;   // element offset of tap (0, 0) in an x plane; may be negative (padding)
+    TT_REQUIRE(e.z % 4 == 0 && e.z >= 0, "%s: pixel table entry %d: x byte offset %d", fn, pq, e.z);
+    for (int r = 0; r < g.R; ++r)
+      for (int s2 = 0; s2 < g.S; ++s2) {
+        const int ih = pp * g.sh - g.ph + r * g.dh, iw = qq * g.sw - g.pw + s2 * g.dw;
+        const bool inside = ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+        const bool blocked = (outside >> (r * g.S + s2)) & 1;
+        TT_REQUIRE(inside != blocked, "%s: pixel table entry %d: tap (%d, %d) at (%d, %d) of a %d x %d image is %s", fn,
+                   pq, r, s2, ih, iw, g.H, g.W, blocked ? "blocked" : "let through");
+        if (!inside) continue;
+        // per column j = (c, r, s) the kernel adds c*H*W + r*dh*W + s*dw elements (jtab)
+        const long long at = first + (long long)r * g.dh * g.W + (long long)s2 * g.dw;
+        TT_REQUIRE(at == (long long)ih * g.W + iw && at + (long long)(Cg - 1) * g.H * g.W < (long long)Cg * g.H * g.W,
+                   "%s: pixel table entry %d: tap (%d, %d) reaches element %lld of its plane (expected %lld)", fn, pq, r, s2,
+                   at, (long long)ih * g.W + iw);
+      }
+  }
+  // per entry: image, sameness with the first image's fields, reach inside both tensors, 31-bit offsets
+  for (int m = 0; m < entries; ++m) {
+    const int4 e = t.tab[(size_t)m];
+    if (m >= M) {
+      TT_REQUIRE(e.x == g.N - 1 && e.y < 0 && mask_of(m) == (wide ? ~0ull : 0xffffffffull),
+                 "%s: pixel table entry %d (past the last pixel) does not read zeros", fn, m);
+      continue;
+    }
+    const int n = m / PQ, pq = m % PQ;
+    const int4 e0 = t.tab[(size_t)pq];
+    TT_REQUIRE(e.x == n && e.y == e0.y && e.z == e0.z && mask_of(m) == mask_of(pq), "%s: pixel table entry %d: image %d, fields differ from pixel %d of image 0", fn, m, e.x, pq);
+    // the chunk's first pixel decides the base image n0 of the descriptors
+    const int n0 = ((m / kBK) * kBK) / PQ;
+    const long long dy_lane = 4LL * (n - n0) * dyImg + e.y + 4LL * (Kg - 1) * PQ;            // last row of a group
+    const long long x_lane = 4LL * (n - n0) * xImg + e.z + 4LL * ((long long)(Cg - 1) * g.H * g.W + (long long)(g.R - 1) * g.dh * g.W + (long long)(g.S - 1) * g.dw);
+    TT_REQUIRE(n >= n0 && dy_lane < (1LL << 31) && x_lane < (1LL << 31),
+               "%s: pixel table entry %d: byte offsets %lld / %lld leave the buffer range", fn, m, dy_lane, x_lane);
+    const long long dy_at = (long long)n * dyImg + (long long)(g.groups - 1) * Kg * PQ + (long long)(Kg - 1) * PQ + pq;
+    TT_REQUIRE(dy_at < (long long)g.N * dyImg, "%s: pixel table entry %d reaches element %lld of dy (%lld)", fn, m, dy_at,
+               (long long)g.N * dyImg);
+  }
+  return 0;
+}
+
+// Set only inside tt_conv2d_check_tables_selftest_wgrad (host-only): damages one field of one
+// entry of the next table built, to show that check_pixtab refuses it.
+int g_pix_fault_entry = -1, g_pix_fault_field = 0, g_pix_fault_delta = 0;
+
 struct PixKey {
-  int v[14];
+  int v[17];
   bool operator<(const PixKey& o) const {
-    for (int i = 0; i < 14; ++i)
+    for (int i = 0; i < 17; ++i)
       if (v[i] != o.v[i]) return v[i] < o.v[i];
     return false;
   }
 };
-// The pixel table depends only on the geometry: built on first use, kept for the process
-// (16 bytes per output pixel, 20 with a 64-bit mask; at most kMaxPixTables geometries, then all are dropped).
+// At most kMaxPixTables geometries (16 bytes per output pixel, 20 with a 64-bit mask), then all are dropped.
 constexpr size_t kMaxPixTables = 256;
 struct PixTables {
-  int4* tab;
-  int* hi;   // null unless the kernel has 32 .. 63 taps
+  int4* tab = nullptr;
+  int* hi = nullptr;   // null unless the kernel has 32 .. 63 taps
+  HostPixTab host;     // stays alive while the upload may still be reading it
 };
 std::map<PixKey, PixTables>& pixtab_cache() {
   static std::map<PixKey, PixTables> cache;
@@ -553,32 +622,45 @@ int drop_pixtabs() {
   cache.clear();
   return 0;
 }
-int cached_pixtab(const Wgrad& p, int N, int P, int Q, bool wide, const int4** out, const int** out_hi) {
+// Builds and checks the table of geometry `g`; unless `host_only`, returns the device copy kept for it.
+int cached_pixtab(const char* fn, const PixGeom& g, bool wide, bool host_only, const int4** out, const int** out_hi) {
   auto& cache = pixtab_cache();
-  const PixKey key{{N, P, Q, p.H, p.W, p.sh, p.sw, p.ph, p.pw, p.dh, p.dw, p.R, p.S, p.chunks}};
-  auto it = cache.find(key);
+  const PixKey key{{g.N, g.C, g.K, g.groups, g.P, g.Q, g.H, g.W, g.R, g.S, g.sh, g.sw, g.ph, g.pw, g.dh, g.dw, g.chunks}};
+  auto it = host_only ? cache.end() : cache.find(key);
   if (it == cache.end()) {
+    PixTables t;
+    build_pixtab(g, wide, &t.host);
+    if (g_pix_fault_entry >= 0 && g_pix_fault_entry < (int)t.host.tab.size()) {   // self-test only
+      int4& e = t.host.tab[(size_t)g_pix_fault_entry];
+      (g_pix_fault_field == 0 ? e.x : g_pix_fault_field == 1 ? e.y : g_pix_fault_field == 2 ? e.z : e.w) ^= g_pix_fault_delta;
+    }
+    if (check_pixtab(fn, g, wide, t.host)) return -1;
+    if (host_only) return 0;
     hipStream_t st = tt::stream();
     if (cache.size() >= kMaxPixTables) {
       TT_HIP(hipStreamSynchronize(st));
       if (drop_pixtabs()) return -1;
     }
-    const int entries = p.chunks * kBK;
-    PixTables t{nullptr, nullptr};
-    TT_HIP(hipMalloc((void**)&t.tab, sizeof(int4) * (size_t)entries));
+    const size_t entries = t.host.tab.size();
+    TT_HIP(hipMalloc((void**)&t.tab, sizeof(int4) * entries));
     if (wide) {
-      if (hipError_t e = hipMalloc((void**)&t.hi, sizeof(int) * (size_t)entries); e != hipSuccess) {
+      if (hipError_t e = hipMalloc((void**)&t.hi, sizeof(int) * entries); e != hipSuccess) {
         (void)hipFree(t.tab);
         return tt::fail_hip(e, "hipMalloc", __FILE__, __LINE__);
       }
     }
-    wgrad_build_pixtab<<<ceil_div(entries, 256), 256, 0, st>>>(t.tab, t.hi, p, entries, N);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
-      (void)hipFree(t.tab);
-      if (t.hi) (void)hipFree(t.hi);
-      return tt::fail_hip(e, "wgrad_build_pixtab", __FILE__, __LINE__);
+    it = cache.emplace(key, std::move(t)).first;   // the vectors' storage moves with it
+    PixTables& kept = it->second;
+    hipError_t e = hipMemcpyAsync(kept.tab, kept.host.tab.data(), sizeof(int4) * entries, hipMemcpyHostToDevice, st);
+    if (e == hipSuccess && wide)
+      e = hipMemcpyAsync(kept.hi, kept.host.hi.data(), sizeof(int) * entries, hipMemcpyHostToDevice, st);
+    if (e != hipSuccess) {
+      (void)hipStreamSynchronize(st);
+      (void)hipFree(kept.tab);
+      if (kept.hi) (void)hipFree(kept.hi);
+      cache.erase(it);
+      return tt::fail_hip(e, "hipMemcpyAsync(pixel table)", __FILE__, __LINE__);
     }
-    it = cache.emplace(key, t).first;
   }
   *out = it->second.tab;
   *out_hi = it->second.hi;
@@ -619,23 +701,43 @@ int wgrad_release_tables() {   // the caller has synchronised the stream
 extern "C" {
 
 // `size_only`: report the workspace bytes this call would ask the library for and do nothing else.
+// `check_only`: build and check the pixel tables the call would use, on the host alone (no device
+// is touched, tensor pointers are not looked at).
 static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
-                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q, size_t* size_only) {
-  TT_REQUIRE_INIT();
+                        int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q, size_t* size_only,
+                        bool check_only = false) {
+  TT_API_LOCK();
   const char* fn = "tt_conv2d_wgrad_f32";
-  TT_REQUIRE(x && dy && dw, "%s: null tensor pointer", fn);
-  TT_REQUIRE_ALIGNED(fn, dw);
+  if (!check_only) {
+    TT_REQUIRE(tt::initialised(), "tt_init() has not been called");
+    TT_REQUIRE(x && dy && dw, "%s: null tensor pointer", fn);
+    TT_REQUIRE_ALIGNED(fn, dw);
+  }
   TT_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0 && P > 0 && Q > 0, "%s: sizes must be positive", fn);
   TT_REQUIRE(sh > 0 && sw > 0 && dh > 0 && dw_ > 0 && ph >= 0 && pw >= 0, "%s: stride/dilation must be positive, padding non-negative", fn);
   TT_REQUIRE(groups > 0 && groups <= 65535 && C % groups == 0 && K % groups == 0, "%s: channels (%d, %d) not divisible by groups=%d", fn, C, K, groups);
   TT_REQUIRE(H + 2 * ph + R * dh < 16384 && W + 2 * pw + S * dw_ < 16384, "%s: spatial extents must stay below 16384", fn);
+  // dy is [N, K, P, Q]: P x Q windows must exist in the padded input.  Fewer than the geometry allows
+  // is legitimate (a transposed convolution with output_padding hands over a cropped problem, as the
+  // reference crops x~ to the rows the windows cover, grad_nn.py:653-655); more is a caller's mix-up
+  // of the roles of x and dy, which would read dy with a wrong pitch and return a plausible dw.
+  {
+    const long long span_h = (long long)H + 2 * ph - (long long)dh * (R - 1) - 1, span_w = (long long)W + 2 * pw - (long long)dw_ * (S - 1) - 1;
+    TT_REQUIRE(span_h >= 0 && span_w >= 0, "%s: kernel (%d x %d, dilation %d x %d) larger than padded input (%d x %d)", fn, R,
+               S, dh, dw_, H + 2 * ph, W + 2 * pw);
+    TT_REQUIRE(P <= span_h / sh + 1 && Q <= span_w / sw + 1,
+               "%s: dy of %d x %d does not belong to this geometry (input %d x %d, kernel %d x %d, stride %d x %d, padding "
+               "%d x %d, dilation %d x %d give at most %lld x %lld)",
+               fn, P, Q, H, W, R, S, sh, sw, ph, pw, dh, dw_, span_h / sh + 1, span_w / sw + 1);
+  }
   // The kernels index with 32-bit element offsets.  A batch whose tensors have 2^31 elements or
   // more is cut into runs of images that stay below that; every run writes its own partial sums
   // and the reduce kernel adds the partials of all runs, still in a fixed order.
   const long long image = std::max((long long)C * H * W, (long long)K * P * Q);
   TT_REQUIRE(tt::fits_i32(image) && tt::fits_i32((long long)K * (C / groups) * R * S),
              "%s: one image or the weights exceed 2^31-1 elements", fn);
-  const int per_run = (int)std::min<long long>(N, std::max<long long>(1, 2147483646LL / image));
+  int per_run = (int)std::min<long long>(N, std::max<long long>(1, 2147483646LL / image));
+  if (per_run < N && per_run >= 4) per_run -= per_run % 4;   // later runs start 16-byte aligned: vector fetches stay on
   const int Cg = C / groups, Kg = K / groups;
   const int J = Cg * R * S;
 
@@ -680,12 +782,12 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     return 0;
   }
   float* target = dw;
-  if (slots > 1) {
+  if (slots > 1 && !check_only) {
     void* ws;
     if (tt::workspace(sizeof(float) * elems * slots, &ws)) return -1;
     target = (float*)ws;
   }
-  hipStream_t st = tt::stream();
+  hipStream_t st = check_only ? nullptr : tt::stream();
   for (const Run& r : runs) {
     Wgrad p{};
     p.x = x + (size_t)r.n0 * C * H * W;
@@ -706,17 +808,17 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     p.outStrideSplit = elems;
     p.R = R; p.S = S;
     p.xBias = ph * W + pw;
-    p.divDh = tt::make_fastdiv((uint32_t)dh);
-    p.divDw = tt::make_fastdiv((uint32_t)dw_);
-    if (R * S <= 31)
-      for (int rr = 0; rr < R; ++rr) p.rowOnes |= 1u << (rr * S);
     // buffer path: byte offsets relative to the first image of a 32-pixel chunk stay below 2 GiB
     // (a chunk spans at most 33 images; x offsets also carry the column's tap and channel offset)
     const long long reach = 4 * (34LL * (p.xStrideN > p.dyStrideN ? p.xStrideN : p.dyStrideN) +
                                  ((long long)H + ph + (long long)R * dh + 2) * W + pw + (long long)S * dw_ + p.xBias);
     const bool buf = R * S <= 63 && reach < (1LL << 31) - (1LL << 20);
     const bool wide = buf && R * S > 31;
-    if (buf && cached_pixtab(p, r.n, P, Q, wide, &p.pixtab, &p.pixhi)) return -1;
+    if (buf) {
+      const PixGeom geom{r.n, C, K, groups, P, Q, H, W, R, S, sh, sw, ph, pw, dh, dw_, r.chunks};
+      if (cached_pixtab(fn, geom, wide, check_only, &p.pixtab, &p.pixhi)) return -1;
+    }
+    if (check_only) continue;
     // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
     const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)p.dy & 15) == 0;
     const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)p.x & 15) == 0;
@@ -734,6 +836,7 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     }
     TT_LAUNCH_CHECK();
   }
+  if (check_only) return 0;
   if (slots > 1) {
     tt::ProfScope prof(TT_PROF_CONV_WGRAD_REDUCE);
     wgrad_reduce<<<ceil_div((long long)elems, 256), kThreads, 0, st>>>(target, dw, elems, slots);
@@ -745,6 +848,38 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
 int tt_conv2d_wgrad_f32(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S,
                         int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
   return conv2d_wgrad(x, dy, dw, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw_, groups, P, Q, nullptr);
+}
+
+// Host-only: builds the pixel tables the call would use for this geometry and checks every entry's
+// reach against x and dy, as the call itself does once per new geometry.
+int tt_conv2d_check_tables_wgrad_f32(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int ph, int pw,
+                                     int dh, int dw_, int groups, int P, int Q) {
+  return conv2d_wgrad(nullptr, nullptr, nullptr, N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw_, groups, P, Q, nullptr, true);
+}
+
+// Host-only: damages single fields of single pixel-table entries (image, dy offset, x offset, a tap
+// bit; 32-bit and 64-bit masks) and returns 0 when the check refuses every damaged table and
+// accepts the undamaged ones.
+int tt_conv2d_check_tables_selftest_wgrad(void) {
+  TT_API_LOCK();
+  struct Case { int R, pad, stride, entry, field, delta; };
+  const Case cases[] = {{3, 1, 1, 7, 0, 1},   {3, 1, 1, 40, 1, 4},  {3, 1, 2, 5, 2, 4},      {3, 1, 1, 0, 3, 1},
+                        {3, 1, 1, 13, 3, 16}, {7, 3, 2, 9, 2, 64},  {7, 3, 2, 30, 3, 1 << 20}, {3, 1, 1, 3 * 144 - 1, 0, 2}};
+  int bad = 0;
+  for (const Case& c : cases) {
+    const int H = 9 + c.R, P = (H + 2 * c.pad - c.R) / c.stride + 1;
+    for (int damaged = 0; damaged < 2; ++damaged) {
+      g_pix_fault_entry = damaged ? c.entry : -1;
+      g_pix_fault_field = c.field;
+      g_pix_fault_delta = c.delta;
+      const int rc = conv2d_wgrad(nullptr, nullptr, nullptr, 3, 8, H, H, 16, c.R, c.R, c.stride, c.stride, c.pad, c.pad, 1, 1, 1,
+                                  P, P, nullptr, true);
+      g_pix_fault_entry = -1;
+      if ((rc != 0) != (damaged != 0)) ++bad;
+    }
+  }
+  TT_REQUIRE(bad == 0, "tt_conv2d_check_tables_selftest_wgrad: %d of 16 table checks gave the wrong verdict", bad);
+  return 0;
 }
 
 int tt_workspace_size_conv2d_wgrad_f32(size_t* bytes, int N, int C, int H, int W, int K, int R, int S, int sh, int sw,

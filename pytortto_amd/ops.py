@@ -10,7 +10,7 @@ from math import prod
 import numpy as np
 
 from . import _hip
-from .xparray import hiparray
+from .xparray import hiparray, poison
 
 
 def _ptr(a):
@@ -116,7 +116,8 @@ class DeferredBatchNorm:
     into ``out``, or into the normalisation's own array when ``out`` is None (an in-place ReLU).
     When the ReLU's result went elsewhere, the normalised values themselves were never stored:
     their array recomputes them (same kernels, same bits, scratch statistics, no running update)
-    should anybody ask for it."""
+    should anybody ask for it, and at the latest just before ``x``, ``gamma`` or ``beta`` is written in
+    place: what is read back is always what the reference stored when the operation ran."""
 
     def __init__(self, x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked):
         self.x, self.gamma, self.beta = x, gamma, beta
@@ -150,8 +151,13 @@ class DeferredBatchNorm:
             scratch = [hiparray.empty((dims[1],)) for _ in range(3)]
             _hip.call('tt_bn_fwd_train_f32', x.ptr, _ptr(gamma), _ptr(beta), buf.ptr, scratch[0].ptr, scratch[1].ptr,
                       scratch[2].ptr, None, None, None, None, None, 0.0, eps, *dims)
-        self.y._buf.on_demand = recompute
+        # x, gamma and beta as they are now: should one of them be written in place later (an
+        # optimiser step, ``+=``), the normalised values are produced first
+        self.y._buf.fill_on_demand(recompute, (x, gamma, beta))
         return out
+
+    def poison(self, exc):
+        poison([self.y, *self.stats, self.new_rm, self.new_rv], exc)
 
 
 def bn_fwd_train_deferred(x, gamma, beta, running_mean, running_var, momentum, eps, num_batches_tracked=None):
@@ -173,6 +179,9 @@ class DeferredReluBackward:
 
     def run(self):
         _hip.call('tt_relu_bwd_f32', self.dy.ptr, self.y.ptr, self.out.ptr, self.y.size)
+
+    def poison(self, exc):
+        poison([self.out], exc)
 
 
 def relu_bwd_deferred(dy, y):
@@ -259,7 +268,8 @@ def add(a, b):
 class DeferredAdd:
     """``a + b`` of equal shapes, not launched yet (see ``_hip.defer``): a ReLU that comes next
     computes ``maximum(a + b, 0)`` in one pass (``run_with_relu``); anything else finds the sum done.
-    When the ReLU's result went to an array of its own, the sum itself is produced on demand."""
+    When the ReLU's result went to an array of its own, the sum itself is produced on demand -- at the
+    latest just before ``a`` or ``b`` is written in place."""
 
     def __init__(self, a, b):
         self.a, self.b = a, b
@@ -274,8 +284,11 @@ class DeferredAdd:
             _hip.call('tt_add_relu_f32', a.ptr, b.ptr, self.out.ptr, a.size)
             return self.out
         _hip.call('tt_add_relu_f32', a.ptr, b.ptr, out.ptr, a.size)
-        self.out._buf.on_demand = lambda buf: _hip.call('tt_add_f32', a.ptr, b.ptr, buf.ptr, a.size)
+        self.out._buf.fill_on_demand(lambda buf: _hip.call('tt_add_f32', a.ptr, b.ptr, buf.ptr, a.size), (a, b))
         return out
+
+    def poison(self, exc):
+        poison([self.out], exc)
 
 
 def add_deferred(a, b):

@@ -26,6 +26,8 @@ def sgd(params, d_p_list, momentum_buffer_list, weight_decay, momentum, lr, damp
         if momentum != 0 and momentum_buffer_list[i] is None:
             momentum_buffer_list[i] = hiparray.empty(param.data.shape)      # the kernel stores d_p into it (:12-13)
             first[i] = 1
+    for param in params:            # written in place: nothing may still depend on the old values
+        param.data.own()
     pointers = ctypes.c_void_p * count
     bufs = pointers(*[None if b is None else b.ptr for b in momentum_buffer_list])
     _hip.call('tt_sgd_step_multi_f32', count, pointers(*[p.data.ptr for p in params]),
@@ -40,6 +42,8 @@ def _adam(params, grads, exp_avgs, exp_avg_sqs, max_exp_avg_sqs, state_steps, am
         return
     for i, param in enumerate(params):
         _device(param, grads[i], exp_avgs[i], exp_avg_sqs[i], max_exp_avg_sqs[i] if amsgrad else None)
+    for param in params:            # written in place: nothing may still depend on the old values
+        param.data.own()
     pointers = ctypes.c_void_p * count
     vmax = pointers(*[a.ptr for a in max_exp_avg_sqs]) if amsgrad else None
     _hip.call('tt_adam_step_multi_f32', count, pointers(*[p.data.ptr for p in params]),

@@ -9,6 +9,7 @@
              an array library.
 """
 import ctypes
+import weakref
 from math import prod
 
 import numpy as np
@@ -59,12 +60,13 @@ class _Buffer:
     that refers to it.  With ``lazy`` the block is taken on the first use of ``ptr``, and
     ``on_demand`` (a callable receiving the buffer) then fills it: the output of an operation that
     was absorbed into its successor exists only if somebody else asks for it."""
-    __slots__ = ('_ptr', 'nbytes', 'on_demand')
+    __slots__ = ('_ptr', 'nbytes', 'on_demand', 'deps', '__weakref__')
 
     def __init__(self, nbytes, lazy=False):
         self.nbytes = nbytes
         self._ptr = 0
         self.on_demand = None
+        self.deps = ()
         if not lazy:
             self._allocate()
 
@@ -73,17 +75,31 @@ class _Buffer:
         _hip.call('tt_malloc', ctypes.byref(p), self.nbytes)
         self._ptr = p.value or 0
 
+    def fill_on_demand(self, fill, operands):
+        """Let ``fill(buffer)`` produce the contents when they are first asked for.  ``operands``
+        are the arrays ``fill`` will read: the reference computed the values when the operation
+        ran, so they must not see a later in-place change of an operand -- ``before_write`` fills
+        this buffer just before any of them is written."""
+        with _hip._lock:
+            self.on_demand = fill
+            self.deps = tuple(a._buf for a in operands if a is not None)
+            _unfilled.add(self)
+
     @property
     def ptr(self):
-        if not self._ptr and self.nbytes:
-            # a parked operation may be the one that produces this very buffer: let it run (and
-            # allocate the buffer itself) before the block is taken here
-            _hip.flush()
-            if not self._ptr:
-                self._allocate()
-        if self.on_demand is not None:
-            fill, self.on_demand = self.on_demand, None
-            fill(self)
+        if (not self._ptr and self.nbytes) or self.on_demand is not None:
+            with _hip._lock:            # two threads may ask for the same unfilled buffer
+                if not self._ptr and self.nbytes:
+                    # a parked operation may be the one that produces this very buffer: let it run
+                    # (and allocate the buffer itself) before the block is taken here
+                    _hip.flush()
+                    if not self._ptr:
+                        self._allocate()
+                if self.on_demand is not None:
+                    fill, self.on_demand = self.on_demand, None
+                    _unfilled.discard(self)
+                    fill(self)
+                    self.deps = ()
         return self._ptr
 
     def __del__(self):
@@ -93,6 +109,32 @@ class _Buffer:
                 self._ptr = 0
         except Exception:   # interpreter shutdown
             pass
+
+
+# buffers whose contents are still to be produced on demand (normally none or a handful: the
+# array of an absorbed BatchNorm or Add output lives only as long as somebody holds its tensor)
+_unfilled = weakref.WeakSet()
+
+
+def before_write(buf):
+    """Called before ``buf`` is overwritten in place: every on-demand buffer that would read it
+    is filled now, from the values the reference's eager evaluation saw."""
+    if not _unfilled:
+        return
+    with _hip._lock:
+        for lazy in list(_unfilled):
+            if any(d is buf for d in lazy.deps):
+                lazy.ptr
+
+
+def poison(arrays, exc):
+    """Make every later use of ``arrays`` raise ``exc``: the operation that was to fill them failed."""
+    def fail(buf):
+        buf.on_demand = fail
+        raise exc
+    for a in arrays:
+        if a is not None:
+            a._buf.on_demand = fail
 
 
 class hiparray:
@@ -214,8 +256,11 @@ class hiparray:
         return other
 
     def own(self):
-        """Make sure this array is the only one on its block before it is written in place."""
-        if self._shared:
+        """Make sure this array is the only one on its block before it is written in place, and
+        that nothing still to be computed on demand depends on the values about to be replaced."""
+        if not self._shared:
+            before_write(self._buf)
+        else:
             fresh = _Buffer(self.nbytes)
             if self.nbytes:
                 _hip.call('tt_memcpy_d2d', fresh.ptr, self._buf.ptr, self.nbytes)

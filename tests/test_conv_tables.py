@@ -1,11 +1,13 @@
-"""Host-only: the index tables behind the convolution forward and input gradient, checked through
-the C ABI without a device (``tt_conv2d_check_tables_*``).
+"""Host-only: the index tables behind the convolution forward, input gradient and weight gradient,
+checked through the C ABI without a device (``tt_conv2d_check_tables_*``).
 
 The kernels address the gathered operand through per-geometry tables (reduction index -> offset
 and tap).  The library builds them on the host and replays every entry for the extreme pixels of
 its tap under the kernel's own bounds rule: the element reached must be the one the reference pairs
 with that reduction index (``grad_nn.py:603-611`` forward, ``:659-682`` input gradient) and lie inside
-the tensor; 32-bit buffer offsets must stay in range.  Here that check runs over the benchmark's
+the tensor; 32-bit buffer offsets must stay in range.  The weight gradient's table has one entry
+per output pixel (``grad_nn.py:646-656``: image, dy offset, x window offset, padding bits), each
+checked tap by tap.  Here that check runs over the benchmark's
 layer shapes at their full batch sizes, the geometries of the GPU parity tests (tile shapes,
 large images, dense few-channel input gradients with every cell size) and seeded random ones.
 """
@@ -35,6 +37,7 @@ def _check_conv(case):
     geo = (r, s, st[0], st[1], pd[0], pd[1], dl[0], dl[1], g)
     _ok(_lib().tt_conv2d_check_tables_fwd_f32(n, c, h, w, k, *geo))
     _ok(_lib().tt_conv2d_check_tables_dgrad_f32(n, c, h, w, k, *geo, p, q))
+    _ok(_lib().tt_conv2d_check_tables_wgrad_f32(n, c, h, w, k, *geo, p, q))
 
 
 def _check_convt(case):
@@ -45,12 +48,32 @@ def _check_convt(case):
     geo = (r, s, st[0], st[1], pd[0], pd[1], dl[0], dl[1], g)
     _ok(_lib().tt_conv2d_check_tables_dgrad_f32(n, co, ho, wo, ci, *geo, h, w))
     _ok(_lib().tt_conv2d_check_tables_fwd_f32(n, co, ho, wo, ci, *geo))     # its input gradient
+    _ok(_lib().tt_conv2d_check_tables_wgrad_f32(n, co, ho, wo, ci, *geo, h, w))   # x := gy, dy := the layer's input
 
 
 def test_table_check_refuses_damaged_tables():
     """Single entries moved by one element, one row or one image, in both addressing modes,
     forward and input gradient: each damaged table is refused, each undamaged one accepted."""
     _ok(_lib().tt_conv2d_check_tables_selftest())
+
+
+def test_pixel_table_check_refuses_damaged_tables():
+    """Weight gradient: a wrong image index, dy offset, x offset or tap bit (let through in the
+    padding, or blocked inside the image) in one entry, 32- and 64-bit masks: each is refused."""
+    _ok(_lib().tt_conv2d_check_tables_selftest_wgrad())
+
+
+def test_weight_gradient_refuses_a_dy_that_does_not_belong_to_the_geometry():
+    """P, Q beyond what (H, R, stride, padding, dilation) allow: the roles of x and dy mixed up."""
+    lib = _lib()
+    geo = (3, 3, 2, 2, 1, 1, 1, 1, 1)
+    _ok(lib.tt_conv2d_check_tables_wgrad_f32(2, 4, 9, 9, 6, *geo, 5, 5))
+    _ok(lib.tt_conv2d_check_tables_wgrad_f32(2, 4, 9, 9, 6, *geo, 4, 5))          # cropped: fewer windows is fine
+    assert lib.tt_conv2d_check_tables_wgrad_f32(2, 4, 9, 9, 6, *geo, 6, 5) != 0
+    assert b'does not belong to this geometry' in lib.tt_last_error()
+    assert lib.tt_conv2d_check_tables_wgrad_f32(2, 4, 9, 9, 6, *geo, 5, 9) != 0
+    assert lib.tt_conv2d_check_tables_wgrad_f32(2, 4, 2, 2, 6, 5, 5, 1, 1, 0, 0, 1, 1, 1, 1, 1) != 0
+    assert b'larger than padded input' in lib.tt_last_error()
 
 
 def test_tables_of_the_benchmark_configurations():
@@ -98,7 +121,7 @@ def test_dense_input_gradient_tables_with_every_cell_size():
         _check_conv((64, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1))
         _check_convt((128, 64, 32, 32, 3, 4, 4, (2, 2), (1, 1), (0, 0), (1, 1), 1))
     finally:
-        _ok(lib.tt_set_conv_dense_cell_min_tiles(384))
+        _ok(lib.tt_set_conv_dense_cell_min_tiles(-1))      # back to the default
 
 
 @pytest.mark.parametrize('seed', [5, 6, 7])

@@ -237,3 +237,106 @@ def _leaf(values):
     import pytortto_amd as tt
     from pytortto_amd.xparray import hiparray
     return tt.Tensor(hiparray(np.ascontiguousarray(values, dtype=np.float32)), requires_grad=True)
+
+
+def test_absorbed_batchnorm_output_read_after_an_optimiser_step_is_the_value_of_the_forward():
+    """y = bn(x); z = relu(y); SGD.step() changes gamma and beta in place; y read afterwards must be what
+    the reference stored when the forward ran (grad_nn.py:952-959), not a recomputation from the new
+    parameters."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn, optim
+    rng = np.random.default_rng(11)
+    x = (1 + 2 * rng.standard_normal((4, 8, 6, 6))).astype(np.float32)
+    gamma, beta = rng.uniform(0.5, 1.5, 8).astype(np.float32), (0.3 * rng.standard_normal(8)).astype(np.float32)
+    bn = nn.BatchNorm2d(8)
+    bn.weight.data[...] = gamma
+    bn.bias.data[...] = beta
+    bn.cuda()
+    y = bn(tt.tensor(x).cuda())
+    z = nn.functional.relu(y)
+    z.backward(tt.tensor(np.ones_like(x)).cuda())
+    optim.SGD(bn.parameters(), lr=0.5).step()
+    assert not np.allclose(bn.weight.data.get(), gamma)               # the step did move the parameters
+    y_ref, _, _, _ = oracle.batch_norm_forward(x, gamma, beta, None, None, True, 0.1, 1e-5)
+    np.testing.assert_allclose(y.data.get(), y_ref, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(z.data.get(), np.maximum(y_ref, 0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize('write', ['iadd_scalar', 'iadd_array', 'fill', 'copy_', 'relu_'])
+def test_absorbed_outputs_are_produced_before_an_operand_is_written_in_place(write):
+    """s = a + b; r = relu(s); a is written in place; s read afterwards equals the a + b of the time the
+    Add ran (autograd/grad_fcn.py:177-203 materialises it then).  The same for bn(x) with x written."""
+    import pytortto_amd as tt
+    from pytortto_amd import nn
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(12)
+    a, b = rng.standard_normal((2, 4, 6, 6)).astype(np.float32), rng.standard_normal((2, 4, 6, 6)).astype(np.float32)
+
+    def overwrite(t):
+        if write == 'iadd_scalar':
+            t.data += 1
+        elif write == 'iadd_array':
+            t.data += hiparray(np.full(a.shape, 2, np.float32))
+        elif write == 'fill':
+            t.data.fill(7.0)
+        elif write == 'copy_':
+            with tt.no_grad():
+                t.copy_(tt.tensor(np.zeros_like(a)))
+        else:
+            nn.functional.relu(t, inplace=True)
+
+    at, bt = tt.Tensor(hiparray(a)), tt.Tensor(hiparray(b))
+    s = at + bt
+    r = nn.functional.relu(s)
+    overwrite(at)
+    assert not np.array_equal(at.data.get(), a)
+    np.testing.assert_array_equal(s.data.get(), a + b)
+    np.testing.assert_array_equal(r.data.get(), np.maximum(a + b, 0))
+
+    x = (1 + 2 * a).astype(np.float32)
+    bn = nn.BatchNorm2d(4)
+    bn.cuda()
+    xt = tt.Tensor(hiparray(x))
+    y = bn(xt)
+    r = nn.functional.relu(y)
+    overwrite(xt)
+    y_ref, _, _, _ = oracle.batch_norm_forward(x, np.ones(4, np.float32), np.zeros(4, np.float32), None, None, True,
+                                               0.1, 1e-5)
+    np.testing.assert_allclose(y.data.get(), y_ref, rtol=1e-5, atol=1e-5)
+
+
+def test_a_parked_operation_is_seen_by_a_second_thread():
+    """Thread B reads the output of an operation thread A parked: it must find it run (one slot shared
+    by all threads, behind a lock), and two threads parking and fusing at once must not mix their ops."""
+    import threading
+    import pytortto_amd as tt
+    from pytortto_amd import _hip, nn, ops
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(13)
+    a, b = rng.standard_normal((64, 33)).astype(np.float32), rng.standard_normal((64, 33)).astype(np.float32)
+    s = tt.Tensor(hiparray(a)) + tt.Tensor(hiparray(b))
+    assert _hip.pending().__class__ is ops.DeferredAdd
+    got = {}
+    t = threading.Thread(target=lambda: got.setdefault('s', s.data.get()))
+    t.start()
+    t.join()
+    np.testing.assert_array_equal(got['s'], a + b)
+
+    errors = []
+
+    def worker(seed):
+        try:
+            r = np.random.default_rng(seed)
+            for _ in range(50):
+                u, v = r.standard_normal((8, 16)).astype(np.float32), r.standard_normal((8, 16)).astype(np.float32)
+                out = nn.functional.relu(tt.Tensor(hiparray(u)) + tt.Tensor(hiparray(v)))
+                np.testing.assert_array_equal(out.data.get(), np.maximum(u + v, 0))
+        except Exception as exc:           # reported by the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors

@@ -127,7 +127,73 @@ def test_conv_dense_input_gradient_with_larger_cells(case):
     try:
         _run_conv(case, seed=3)
     finally:
-        _hip.call('tt_set_conv_dense_cell_min_tiles', 384)
+        _hip.call('tt_set_conv_dense_cell_min_tiles', -1)        # back to the default
+
+
+STREAM_K_CASES = [c for c in TILE_CASES if c[:3] in ((8, 128, 28), (16, 64, 56), (16, 256, 14))]
+
+
+def _last_launch():
+    import ctypes
+    from pytortto_amd import _hip
+    plan = (ctypes.c_int * 8)()
+    _hip.call('tt_conv2d_last_launch', plan)
+    return dict(zip(('bm', 'bn', 'tiles', 'tiles_i', 'persistent_blocks', 'whole_tiles', 'sharing_blocks', 'mode'), plan))
+
+
+def test_persistent_grid_kernels_fit_the_device():
+    """The blocks of a persistent launch wait for each other's partial sums; that is safe only while
+    two blocks (three with bf16 arithmetic) of every such kernel are resident per compute unit."""
+    import ctypes
+    from pytortto_amd import _hip
+    held = ctypes.c_int()
+    _hip.call('tt_conv2d_stream_k_blocks_per_cu', 0, ctypes.byref(held))
+    assert held.value >= 2, held.value
+    _hip.call('tt_conv2d_stream_k_blocks_per_cu', 1, ctypes.byref(held))
+    assert held.value >= 3, held.value
+
+
+@pytest.mark.parametrize('case', STREAM_K_CASES)
+def test_persistent_grid_falls_back_to_one_tile_per_block_when_it_would_not_fit(case):
+    """With the device reporting (here: made to report) one resident block per compute unit, the
+    launches that would share reductions between blocks run data-parallel, and still match."""
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    assert len(STREAM_K_CASES) == 3
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(9)
+    x = hiparray(rng.standard_normal((n, c, h, w_)).astype(np.float32))
+    w = hiparray((rng.standard_normal((k, c // g, r, s)) / np.sqrt(c // g * r * s)).astype(np.float32))
+    y_shared = ops.conv2d_fwd(x, w, None, st, pd, dl, g).get()
+    assert _last_launch()['persistent_blocks'] > 0 and _last_launch()['sharing_blocks'] > 0
+    _hip.call('tt_conv2d_stream_k_force_occupancy', 1)
+    try:
+        y_plain = ops.conv2d_fwd(x, w, None, st, pd, dl, g).get()
+        plan = _last_launch()
+        assert plan['persistent_blocks'] == 0 and plan['whole_tiles'] == plan['tiles']
+        _run_conv(case, seed=2)
+    finally:
+        _hip.call('tt_conv2d_stream_k_force_occupancy', -1)
+    np.testing.assert_allclose(y_plain, y_shared, rtol=1e-5, atol=1e-5)     # summation order of the shared tiles only
+
+
+def test_a_wait_that_ran_out_is_reported_by_the_next_synchronisation():
+    """Host side of the failure path: the word a block sets when its bounded wait runs out (set here by
+    a one-thread kernel; nothing waits) makes the next tt_sync / device-to-host copy fail with the
+    documented message, once; afterwards the library works as before."""
+    from pytortto_amd import _hip
+    from pytortto_amd.xparray import hiparray
+    _hip.synchronize()
+    _hip.call('tt_conv2d_selftest_raise_async_error')
+    with pytest.raises(RuntimeError, match='timed out waiting for another block'):
+        _hip.synchronize()
+    _hip.synchronize()                                  # reported once, then clear
+    a = hiparray(np.arange(8, dtype=np.float32))
+    _hip.call('tt_conv2d_selftest_raise_async_error')
+    with pytest.raises(RuntimeError, match='results since the last synchronisation are invalid'):
+        a.get()
+    np.testing.assert_array_equal(a.get(), np.arange(8, dtype=np.float32))
+    _run_conv(STREAM_K_CASES[0], seed=4)
 
 
 # Images too large for 32-bit byte offsets relative to a tile's (a chunk's) first image: the

@@ -210,3 +210,97 @@ def test_checkpoint_wire_format_round_trip(tmp_path):
         np.testing.assert_array_equal(v, sd[k])
     with pytest.raises(RuntimeError, match='Missing key'):
         other.load_state_dict({k: v for k, v in sd.items() if k != '1.running_var'})
+
+
+def test_host_relu_while_a_device_operation_is_parked(monkeypatch):
+    """A host ReLU must not look for a device buffer on its input: with a device BatchNorm or Add
+    still parked, relu(host tensor) takes tortto's NumPy expression and leaves the parked operation
+    alone.  (Stand-ins for the parked objects: nothing here touches a GPU.)"""
+    from pytortto_amd import _hip, ops
+
+    class _Out:
+        _buf = object()
+
+    for cls, field in ((ops.DeferredBatchNorm, 'y'), (ops.DeferredAdd, 'out')):
+        fake = object.__new__(cls)
+        setattr(fake, field, _Out())
+        monkeypatch.setattr(_hip, '_pending', fake)
+        for inplace in (False, True):
+            x = tt.tensor(np.array([-1.0, 2.0, -3.0], np.float32))
+            y = tt.nn.functional.relu(x, inplace=inplace)
+            np.testing.assert_array_equal(y.data, np.array([0.0, 2.0, 0.0], np.float32))
+        assert _hip.pending() is fake
+    monkeypatch.setattr(_hip, '_pending', None)
+
+
+def test_parked_operation_slot_is_atomic_and_poisons_on_failure():
+    """take_pending_if tests and takes in one step; an operation that fails when it is flushed marks
+    its outputs so that they raise instead of handing out memory nobody wrote."""
+    from pytortto_amd import _hip
+    from pytortto_amd.xparray import poison
+
+    class Op:
+        ran = 0
+
+        def run(self):
+            Op.ran += 1
+
+    op = Op()
+    _hip.defer(op)
+    assert _hip.take_pending_if(lambda o: False) is None and _hip.pending() is op
+    assert _hip.take_pending_if(lambda o: o is op) is op and _hip.pending() is None
+    _hip.defer(op)
+    _hip.flush()
+    assert Op.ran == 1 and _hip.pending() is None
+
+    class Buf:
+        on_demand = None
+
+    class Arr:
+        def __init__(self):
+            self._buf = Buf()
+
+    class Failing:
+        def __init__(self):
+            self.out = Arr()
+
+        def run(self):
+            raise RuntimeError('shape limit')
+
+        def poison(self, exc):
+            poison([self.out, None], exc)
+
+    bad = Failing()
+    _hip.defer(bad)
+    with pytest.raises(RuntimeError, match='shape limit'):
+        _hip.flush()
+    assert _hip.pending() is None
+    for _ in range(2):                      # stays poisoned
+        with pytest.raises(RuntimeError, match='shape limit'):
+            bad.out._buf.on_demand(bad.out._buf)
+
+
+def test_runs_of_a_long_batch_start_aligned():
+    """Batches of 2^31 elements or more are cut into runs of images; every run but the first starts
+    `per` images in, and the kernels need 16-byte aligned pointers: per * image must be a multiple of
+    four elements for both tensors, whatever the image sizes."""
+    import ctypes
+    from pytortto_amd import _hip
+    lib = _hip.load_library()
+
+    def per_run(n, a, b):
+        out = ctypes.c_int()
+        assert lib.tt_conv2d_images_per_run(n, a, b, ctypes.byref(out)) == 0
+        return out.value
+
+    assert per_run(64, 3 * 224 * 224, 64 * 112 * 112) == 64              # fits: one run
+    for image_a, image_b in [(2 ** 20, 2 ** 20), (3 * 333 * 333, 5 * 167 * 167), (7 * 1001 * 999, 3 * 501 * 500),
+                             (1000003, 999983), (2 ** 20 + 2, 2 ** 19 + 1), (2 ** 30 + 1, 5)]:
+        n = 3 * (2 ** 31) // max(image_a, image_b) + 7
+        per = per_run(n, image_a, image_b)
+        if per == 0:        # only when not even one image keeps the runs aligned
+            assert max(image_a, image_b) * 4 > 2 ** 31 - 2 and (image_a % 4 or image_b % 4)
+            continue
+        assert 1 <= per < n and per * max(image_a, image_b) < 2 ** 31
+        assert (per * image_a) % 4 == 0 and (per * image_b) % 4 == 0, (per, image_a, image_b)
+        assert (per + 4) * max(image_a, image_b) >= 2 ** 31 - 1            # not needlessly short
