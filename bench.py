@@ -43,14 +43,66 @@ RESNET50_CONVS = [
     (512, 7, 2048, 1, 1, 0, 3), (2048, 7, 512, 1, 1, 0, 2), (512, 7, 512, 3, 1, 1, 2),
 ]
 BATCH = 64
-# HBM bytes per launch of the two dominant kernels, from rocprofv3 FETCH_SIZE + WRITE_SIZE of this
-# workload (each counter scaled by what it reads for the 2 GiB copy probe of the same run: x2.0 and
-# x1.0).  Counters cannot be read from inside this script, so the figures of the last counter
-# run are carried here; the summary with the commands is in the profiles directory
-# (bench_hbm_traffic_fetch_write_size.txt).
-IGEMM_TRAFFIC_BYTES_PER_LAUNCH = 170.0e6      # igemm_f32 + igemm_multi_f32, mean over the 106 launches of a step (106.9e6 algorithmic)
-BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH = 925.2e6   # mean of the two shapes (3*S = 924.8e6 algorithmic)
-MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH = 311.7e6    # dy + taps read, dx written (308.3e6 algorithmic)
+# HBM bytes per launch of the dominant kernels come from rocprofv3 FETCH_SIZE + WRITE_SIZE runs of this
+# workload (each counter scaled by what it reads for the 2 GiB copy probe of the same run).  Counters
+# cannot be read from inside this script, so the figures are read from the committed summary of the
+# last counter run, a table keyed on the kernel instantiation name that also records the hashes of
+# the kernel sources it was taken with: a kernel that was renamed is not found, and sources that
+# changed since make the figure stale -- both give `traffic: null` with the reason beside it.
+TRAFFIC_SUMMARY = os.path.join(ROOT, 'profiles', 'bench_hbm_traffic_fetch_write_size.txt')
+BRACKETED_IGEMM_LAUNCHES_PER_STEP = 106       # forward + input gradient of the 53 layers
+
+
+def _sha16(path):
+    import hashlib
+    with open(path, 'rb') as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def traffic_table(path=TRAFFIC_SUMMARY):
+    """({kernel name: (dispatches, bytes per dispatch)}, conv steps in the counter run, None or why the
+    table cannot be used)."""
+    import re
+    rows, steps, sources = {}, None, {}
+    try:
+        with open(path) as f:
+            for line in f:
+                m = re.match(r'^(\S.*?)\s{2,}(\d+)\s+([\d.]+)\s+([\d.]+)\s+([\d.]+)\s*$', line)
+                if m:
+                    rows[m.group(1).strip()] = (int(m.group(2)), float(m.group(5)) * 1e6)
+                m = re.match(r'^kernel source (\S+) sha256 (\w+)', line)
+                if m:
+                    sources[m.group(1)] = m.group(2)
+                m = re.match(r'^conv steps per precision in each run: (\d+)', line)
+                if m:
+                    steps = int(m.group(1))
+    except OSError as exc:
+        return {}, None, f'no counter summary ({exc})'
+    if not rows or not steps or not sources:
+        return rows, steps, 'the counter summary holds no table, step count or source hashes'
+    for name, sha in sources.items():
+        src = os.path.join(ROOT, 'pytortto_amd', 'csrc', name)
+        if not os.path.exists(src) or _sha16(src) != sha:
+            return rows, steps, f'stale: {name} changed since the counter run'
+    return rows, steps, None
+
+
+def traffic_per_launch(prefixes, launches_per_step=None):
+    """Bytes per launch of the kernels whose instantiation names start with one of `prefixes`: the
+    mean over their dispatches, or -- with `launches_per_step` -- their bytes per step divided by
+    that many bracketed launches.  (None, reason) when the table cannot serve it."""
+    rows, steps, why = traffic_table()
+    if why:
+        return None, why
+    hit = {n: v for n, v in rows.items() if any(n == p or n.startswith(p + '<') for p in prefixes)}
+    if not hit:
+        return None, f'no kernel named {" / ".join(prefixes)} in the counter summary'
+    total = sum(d * b for d, b in hit.values())
+    if launches_per_step:
+        return total / (steps * launches_per_step), None
+    return total / sum(d for d, _ in hit.values()), None
+
+
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
 
 
@@ -76,12 +128,59 @@ class ConvLayer:
         self.dw = hiparray.empty((k, c, r, r))
         self.args = (batch, c, h, h, k, r, r, s, s, p, p, 1, 1, 1)
         self.q = q
+        self.label = f'{c}x{h}x{h}->{k} k{r} s{s} p{p}'
+        self.nbytes = 4.0 * (self.x.size + self.w.size + self.y.size)
+
+    def passes(self, call):
+        a = self.args
+        return {'fwd': lambda: call('tt_conv2d_fwd_f32', self.x.ptr, self.w.ptr, None, self.y.ptr, *a),
+                'dgrad': lambda: call('tt_conv2d_dgrad_f32', self.dy.ptr, self.w.ptr, None, self.dx.ptr, *a, self.q, self.q),
+                'wgrad': lambda: call('tt_conv2d_wgrad_f32', self.x.ptr, self.dy.ptr, self.dw.ptr, *a, self.q, self.q)}
 
     def run(self, call):
         a = self.args
         call('tt_conv2d_fwd_f32', self.x.ptr, self.w.ptr, None, self.y.ptr, *a)
         call('tt_conv2d_dgrad_f32', self.dy.ptr, self.w.ptr, None, self.dx.ptr, *a, self.q, self.q)
         call('tt_conv2d_wgrad_f32', self.x.ptr, self.dy.ptr, self.dw.ptr, *a, self.q, self.q)
+
+
+# PreAct-ResNet-18 basic-block stack on 3x32x32 inputs: the 11 unique convolution shapes, as RESNET50_CONVS
+PREACT18_CONVS = [(3, 32, 64, 3, 1, 1, 1), (64, 32, 64, 3, 1, 1, 4), (64, 32, 128, 3, 2, 1, 1), (128, 16, 128, 3, 1, 1, 3),
+                  (64, 32, 128, 1, 2, 0, 1), (128, 16, 256, 3, 2, 1, 1), (256, 8, 256, 3, 1, 1, 3), (128, 16, 256, 1, 2, 0, 1),
+                  (256, 8, 512, 3, 2, 1, 1), (512, 4, 512, 3, 1, 1, 3), (256, 8, 512, 1, 2, 0, 1)]
+# DCGAN generator: (C_in, H_in, C_out, kernel, stride, padding) of the five ConvTranspose2d layers
+DCGAN_CONVTS = [(100, 1, 512, 4, 1, 0), (512, 4, 256, 4, 2, 1), (256, 8, 128, 4, 2, 1), (128, 16, 64, 4, 2, 1),
+                (64, 32, 3, 4, 2, 1)]
+
+
+class ConvTransposeLayer:
+    """One ConvTranspose2d shape: its forward is the input-gradient call of the convolution with the
+    same geometry, its input gradient that convolution's forward call, its weight gradient the
+    weight-gradient call with the roles of x and dy exchanged (grad_nn.py:755, :776-778).  Useful
+    FLOPs per pass: 2*N*C_in*C_out*R*S*H_in*W_in (the reference's zero-insertion executes stride^2
+    times that)."""
+
+    def __init__(self, spec, batch, rng):
+        from pytortto_amd.xparray import hiparray
+        ci, h, co, r, st, pd = spec
+        ho = (h - 1) * st - 2 * pd + (r - 1) + 1
+        self.spec, self.count, self.batch = spec, 1, batch
+        self.flops = 2.0 * batch * ci * co * r * r * h * h
+        bound = 1.0 / np.sqrt(co * r * r)
+        self.x = hiparray(rng.standard_normal((batch, ci, h, h), dtype=np.float32))
+        self.w = hiparray(rng.uniform(-bound, bound, (ci, co, r, r)).astype(np.float32))
+        self.g = hiparray(rng.standard_normal((batch, co, ho, ho), dtype=np.float32))
+        self.y, self.dx, self.dw = hiparray.empty((batch, co, ho, ho)), hiparray.empty((batch, ci, h, h)), hiparray.empty((ci, co, r, r))
+        self.args = (batch, co, ho, ho, ci, r, r, st, st, pd, pd, 1, 1, 1)
+        self.h = h
+        self.label = f'{ci}x{h}x{h}->{co}x{ho}x{ho} k{r} s{st} p{pd} (transposed)'
+        self.nbytes = 4.0 * (self.x.size + self.w.size + self.y.size)
+
+    def passes(self, call):
+        a, h = self.args, self.h
+        return {'fwd': lambda: call('tt_conv2d_dgrad_f32', self.x.ptr, self.w.ptr, None, self.y.ptr, *a, h, h),
+                'dgrad': lambda: call('tt_conv2d_fwd_f32', self.g.ptr, self.w.ptr, None, self.dx.ptr, *a),
+                'wgrad': lambda: call('tt_conv2d_wgrad_f32', self.g.ptr, self.x.ptr, self.dw.ptr, *a, h, h)}
 
 
 class BnLayer:
@@ -186,31 +285,74 @@ def profiled_steps(hip, step, steps):
 
 
 def per_layer_table(hip, call, layers, reps):
-    """Forward, input gradient and weight gradient of every unique ResNet-50 shape timed on their own
+    """Forward, input gradient and weight gradient of every unique shape timed on their own
     (HIP events on the library stream around `reps` back-to-back calls after 3 warm-up calls; the
     weight gradient includes its float64 reduce, the input gradient its weight repack).  The
     per-layer roofline is min(fp32 MFMA peak, AI * 8 TB/s) with AI = F / (4 * (|x| + |w| + |y|)):
     the three passes of a layer move the same three tensors' worth of bytes."""
     rows = []
     for l in layers:
-        c, h, k, r, s, p, count = l.spec
-        a = l.args
-        passes = {
-            'fwd': lambda: call('tt_conv2d_fwd_f32', l.x.ptr, l.w.ptr, None, l.y.ptr, *a),
-            'dgrad': lambda: call('tt_conv2d_dgrad_f32', l.dy.ptr, l.w.ptr, None, l.dx.ptr, *a, l.q, l.q),
-            'wgrad': lambda: call('tt_conv2d_wgrad_f32', l.x.ptr, l.dy.ptr, l.dw.ptr, *a, l.q, l.q),
-        }
-        nbytes = 4.0 * (l.x.size + l.w.size + l.y.size)
-        ai = l.flops / nbytes
+        ai = l.flops / l.nbytes
         roof = min(PEAK_FP32_MFMA_TFLOPS, ai * PEAK_HBM_GBS / 1e3)
-        row = {'shape': f'{c}x{h}x{h}->{k} k{r} s{s} p{p}', 'count': count, 'gflop': round(l.flops / 1e9, 2),
+        row = {'shape': l.label, 'count': l.count, 'gflop': round(l.flops / 1e9, 3),
                'ai_flop_per_byte': round(ai, 1), 'roofline_tflops': round(roof, 1)}
-        for name, fn in passes.items():
+        for name, fn in l.passes(call).items():
             ms, _ = timed_steps(hip, fn, reps, 3)
             tf = l.flops / (ms * 1e-3) / 1e12
             row[name] = {'ms': round(ms, 4), 'tflops': round(tf, 1), 'frac_of_roofline': round(tf / roof, 3)}
         rows.append(row)
     return rows
+
+
+def table_totals(rows):
+    """Time and rate of one step made of the rows' passes (every occurrence of every shape)."""
+    ms = sum(r['count'] * (r['fwd']['ms'] + r['dgrad']['ms'] + r['wgrad']['ms']) for r in rows)
+    gflop = sum(3 * r['count'] * r['gflop'] for r in rows)
+    return {'layers_ms_summed': round(ms, 3), 'gflop': round(gflop, 2), 'tflops': round(gflop / ms, 2),
+            'frac_of_fp32_mfma_peak': round(gflop / ms / PEAK_FP32_MFMA_TFLOPS, 4)}
+
+
+def single_layer_config(hip, call, rng, reps=200):
+    """The CPU-runnable baseline configuration on the GPU: Conv2d(16, 32, 3, padding=1, bias) on
+    x [32,16,32,32], forward (with bias), input gradient, weight gradient and bias gradient.  At 0.3
+    GFLOP per pass every call is one launch of a few microseconds: the figures are bound by launch
+    and ramp-up, not by the matrix pipe, and say so."""
+    from pytortto_amd.xparray import hiparray
+    x = hiparray(rng.standard_normal((32, 16, 32, 32), dtype=np.float32))
+    w = hiparray(rng.uniform(-1 / 12, 1 / 12, (32, 16, 3, 3)).astype(np.float32))
+    b = hiparray(rng.uniform(-1 / 12, 1 / 12, 32).astype(np.float32))
+    dy = hiparray(rng.standard_normal((32, 32, 32, 32), dtype=np.float32))
+    y, dx, dw, db = hiparray.empty(dy.shape), hiparray.empty(x.shape), hiparray.empty(w.shape), hiparray.empty((32,))
+    a = (32, 16, 32, 32, 32, 3, 3, 1, 1, 1, 1, 1, 1, 1)
+    flops = 2.0 * 32 * 32 * 16 * 9 * 32 * 32
+    nbytes = 4.0 * (x.size + w.size + y.size)
+    roof = min(PEAK_FP32_MFMA_TFLOPS, flops / nbytes * PEAK_HBM_GBS / 1e3)
+    passes = {'fwd': lambda: call('tt_conv2d_fwd_f32', x.ptr, w.ptr, b.ptr, y.ptr, *a),
+              'dgrad': lambda: call('tt_conv2d_dgrad_f32', dy.ptr, w.ptr, None, dx.ptr, *a, 32, 32),
+              'wgrad': lambda: call('tt_conv2d_wgrad_f32', x.ptr, dy.ptr, dw.ptr, *a, 32, 32),
+              'bias_grad': lambda: call('tt_channel_sum_f32', dy.ptr, db.ptr, 32, 32, 1024)}
+    out = {'config': {'workload': 'Conv2d(16, 32, 3, padding=1, bias) on x [32,16,32,32], fwd + dgrad + wgrad + bias gradient; '
+                                  '0.302 GFLOP per pass'},
+           'roofline_tflops': round(roof, 1), 'ai_flop_per_byte': round(flops / nbytes, 1)}
+    total = 0.0
+    for name, fn in passes.items():
+        ms, _ = timed_steps(hip, fn, reps, 10)
+        total += ms
+        out[name] = {'ms': round(ms, 5)}
+        if name != 'bias_grad':
+            tf = flops / (ms * 1e-3) / 1e12
+            out[name].update(tflops=round(tf, 2), frac_of_roofline=round(tf / roof, 3))
+
+    def whole():
+        for fn in passes.values():
+            fn()
+    ms, wall = timed_steps(hip, whole, reps, 10)
+    tf = 3 * flops / (ms * 1e-3) / 1e12
+    out.update(value=round(tf, 2), unit='TFLOP/s', ms_per_step=round(ms, 5), wall_ms_per_step=round(wall, 5),
+               frac_of_roofline=round(tf / roof, 3),
+               note='launch-bound: each pass is one to three kernels of 5-15 us; back-to-back launches overlap their ramp-up, '
+                    'so the step is shorter than the sum of the passes timed alone')
+    return out
 
 
 def resnet50_train_step(hip, steps, warmup, batch=BATCH):
@@ -384,7 +526,7 @@ def cpu_threads():
 
 
 def cpu_baseline_conv(batch):
-    """Oracle fwd + dgrad + wgrad, once per unique ResNet-50 shape, at a reduced batch."""
+    """Oracle fwd + dgrad + wgrad, once per unique ResNet-50 shape, at the given batch."""
     import oracle
     rng = np.random.default_rng(0)
     flops = 0.0
@@ -446,6 +588,9 @@ def main():
     ap.add_argument('--steps', type=int, default=10)
     ap.add_argument('--warmup', type=int, default=3)
     ap.add_argument('--no-cpu-baseline', action='store_true', help='skip the host-side oracle timing')
+    ap.add_argument('--cpu-batch', type=int, default=BATCH,
+                    help='batch of the CPU baseline over the 23 ResNet-50 shapes (default: the benchmark batch, 64; '
+                         'about 2.5 minutes of host time)')
     ap.add_argument('--no-model-step', action='store_true', help='skip the whole-network ResNet-50 training step')
     ap.add_argument('--model-step-only', action='store_true',
                     help='run only the whole-network ResNet-50 training step and print its object (for profiling)')
@@ -527,6 +672,7 @@ def main():
     wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
     kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
     layer_rows = None if args.no_per_layer else per_layer_table(_hip, call, layers, 20)
+    c1_gpu = single_layer_config(_hip, call, rng)
 
     # optional reduced-precision variant, reported separately and never part of `value`: the three
     # passes on bf16 MFMA (operands rounded inside the kernels, fp32 accumulation and tensors)
@@ -635,7 +781,16 @@ def main():
                                         'loss_first_last': [round(b_losses[0], 4), round(b_losses[-1], 4)]}
         call('tt_empty_cache')
 
-    # ---- the other two stack configurations, through the module API -----------------------------
+    # ---- the other two stack configurations: per layer, then whole stacks through the module API ---
+    stack_rows = {}
+    if not args.no_per_layer:
+        for key, cls, specs in (('preact_resnet18_stack', ConvLayer, PREACT18_CONVS),
+                                ('dcgan_generator_stack', ConvTransposeLayer, DCGAN_CONVTS)):
+            ls = [cls(spec, 128, rng) for spec in specs]
+            rows = per_layer_table(_hip, call, ls, 30)
+            stack_rows[key] = {'rows': rows, 'all_layers': table_totals(rows)}
+            del ls
+            call('tt_empty_cache')
     stacks = None
     if not args.no_model_step:
         # steps of 1-6 ms: enough of them that the first ones (pool refill after tt_empty_cache, clock
@@ -651,25 +806,36 @@ def main():
                       'metric': 'PreAct-ResNet-18 basic-block stack fwd+bwd (conv + BatchNorm + ReLU + shortcuts)',
                       'config': {'workload': 'batch 128, 3x32x32, 20 convolutions, 142.19 GFLOP per pass'},
                       'ms_per_step': round(p_wall, 3), 'gpu_ms_per_step': round(p_ms, 3),
-                      'conv_tflops_equivalent': round(3 * 142.19e9 / (p_wall * 1e-3) / 1e12, 2)},
+                      'conv_tflops_equivalent': round(3 * 142.19e9 / (p_wall * 1e-3) / 1e12, 2),
+                      'per_layer': stack_rows.get('preact_resnet18_stack')},
                   'dcgan_generator_stack': {
                       'metric': 'DCGAN generator fwd+bwd (ConvTranspose2d + BatchNorm + ReLU)',
                       'config': {'workload': 'batch 128, latent 100 -> 3x64x64, 5 transposed convolutions, '
                                              '26.78 GFLOP per pass'},
                       'ms_per_step': round(d_wall, 3), 'gpu_ms_per_step': round(d_ms, 3),
-                      'conv_tflops_equivalent': round(3 * 26.78e9 / (d_wall * 1e-3) / 1e12, 2)},
+                      'conv_tflops_equivalent': round(3 * 26.78e9 / (d_wall * 1e-3) / 1e12, 2),
+                      'per_layer': stack_rows.get('dcgan_generator_stack')},
                   'note': 'whole stacks, every kernel counted in the time, only convolution FLOPs in the rate; '
-                          'the input of the first layer needs no gradient, so its input-gradient pass does not run'}
+                          'the input of the first layer needs no gradient, so its input-gradient pass does not run.  '
+                          'per_layer: every unique convolution shape of the stack at batch 128 timed alone (30 calls '
+                          'after 3 warm-up calls), each with its own roofline min(157.3, AI * 8 TB/s); transposed '
+                          'layers count useful FLOPs 2*N*C_in*C_out*R*S*H_in*W_in'}
+    elif stack_rows:
+        stacks = {k: {'per_layer': v} for k, v in stack_rows.items()}
 
     # ---- CPU baseline (oracle on the host cores) -------------------------------------------------
     cpu_conv = cpu_bn = None
     if not args.no_cpu_baseline:
         cores = cpu_threads()
-        cbatch = 8
-        f, sec = cpu_baseline_conv(cbatch)
+        f, sec = cpu_baseline_conv(args.cpu_batch)
         cpu_conv = {'value': round(f / sec / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
                     'sample': f'oracle fwd+dgrad+wgrad once over the 23 unique ResNet-50 conv shapes at batch '
-                              f'{cbatch} ({f / 1e9:.0f} GFLOP counted, {sec:.1f} s)'}
+                              f'{args.cpu_batch}{" (the benchmark batch)" if args.cpu_batch == BATCH else ""} '
+                              f'({f / 1e9:.0f} GFLOP counted, {sec:.1f} s, one repetition per shape)'}
+        if args.cpu_batch != 8:
+            f8, sec8 = cpu_baseline_conv(8)
+            cpu_conv['at_batch_8'] = {'value': round(f8 / sec8 / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
+                                      'sample': f'the same 23 shapes at batch 8 ({f8 / 1e9:.0f} GFLOP counted, {sec8:.1f} s)'}
         f1, sec1 = cpu_baseline_c1()
         cpu_conv['single_layer_config_full_size'] = {
             'value': round(f1 / sec1 / 1e12, 4), 'unit': 'TFLOP/s', 'cores': cores, 'kind': 'port',
@@ -680,6 +846,9 @@ def main():
                   'sample': f'oracle BatchNorm fwd+bwd at both shapes, full batch ({nb / 1e9:.2f} GB counted, '
                             f'{sec:.1f} s)'}
 
+    igemm_traffic, igemm_traffic_why = traffic_per_launch(('igemm_f32', 'igemm_multi_f32'), BRACKETED_IGEMM_LAUNCHES_PER_STEP)
+    bn_traffic, bn_traffic_why = traffic_per_launch(('bn_bwd_apply',))
+    pool_traffic, pool_traffic_why = traffic_per_launch(('maxpool_bwd_scatter',))
     out = {
         'metric': 'conv fwd+bwd TFLOP/s (% fp32 MFMA peak); BatchNorm2d fwd+bwd GB/s (% HBM)',
         'value': round(conv_tflops, 2), 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -693,7 +862,7 @@ def main():
         'roofline': {'bound': 'mfma', 'kernel': 'igemm_f32 (Conv2d forward + input gradient)',
                      'achieved': round(igemm_tflops, 2), 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(igemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
-                     'traffic': IGEMM_TRAFFIC_BYTES_PER_LAUNCH,
+                     'traffic': igemm_traffic, 'traffic_note': igemm_traffic_why,
                      'sustained_peak_measured': {'mean': round(mfma_mean, 1), 'min': round(mfma_min, 1),
                                                  'max': round(mfma_max, 1), 'unit': 'TFLOP/s',
                                                  'what': '100 launches of dense v_mfma_f32_32x32x2_f32, '
@@ -707,6 +876,7 @@ def main():
                       'rows': layer_rows},
         'conv_bf16_variant': bf16_variant,
         'cpu_baseline': cpu_conv,
+        'single_layer_config': c1_gpu,
         'bn': {'metric': 'BatchNorm2d training fwd+bwd GB/s', 'value': round(bn_gbs, 1), 'unit': 'GB/s',
                'ms_per_step': round(bn_ms, 4), 'wall_ms_per_step': round(bn_wall_ms, 4),
                'pct_of_peak': round(100 * bn_gbs / PEAK_HBM_GBS, 1),
@@ -720,7 +890,7 @@ def main():
                'roofline': {'bound': 'hbm', 'kernel': 'bn_bwd_apply (reads x, dy; writes dx)',
                             'achieved': round(bwd_apply_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                             'frac': round(bwd_apply_gbs / PEAK_HBM_GBS, 4),
-                            'traffic': BN_BWD_APPLY_TRAFFIC_BYTES_PER_LAUNCH,
+                            'traffic': bn_traffic, 'traffic_note': bn_traffic_why,
                             'sustained_measured': {'read_gbs': round(hbm_read, 1), 'copy_gbs': round(hbm_copy, 1),
                                                    'what': '2 GiB streamed, 16 KiB contiguous per block'},
                             'avg_launch_ms': round(ms_ba / max(1, n_ba), 5)},
@@ -734,7 +904,7 @@ def main():
                     'roofline': {'bound': 'hbm', 'kernel': 'maxpool_bwd_scatter (reads dy, taps; writes dx)',
                                  'achieved': round(pool_bwd_gbs, 1), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                                  'frac': round(pool_bwd_gbs / PEAK_HBM_GBS, 4),
-                                 'traffic': MAXPOOL_BWD_TRAFFIC_BYTES_PER_LAUNCH,
+                                 'traffic': pool_traffic, 'traffic_note': pool_traffic_why,
                                  'avg_launch_ms': round(ms_pb / max(1, n_pb), 5)},
                     'kernels_ms_per_step': {'maxpool_fwd': round(ms_pf / max(1, n_pf), 4),
                                             'maxpool_bwd': round(ms_pb / max(1, n_pb), 4)},

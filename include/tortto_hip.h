@@ -202,6 +202,14 @@ int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* p
  * grid (0 = one tile per block), tiles computed whole, blocks sharing the remaining tiles'
  * reductions, addressing mode.  Tests use it to compare the images where the shared tiles begin. */
 int tt_conv2d_last_launch(int* plan8);
+/* The same for the weight gradient, whose blocks add each other's partial sums inside the kernel
+ * when the device holds the whole grid at once and leave them to a second kernel otherwise:
+ *   tt_conv2d_last_wgrad_launch: {tiles, reduction splits, 1 if added inside the kernel, partial-sum
+ *     slots} of the last launch (host pointer to 4 ints);
+ *   tt_conv2d_wgrad_force_occupancy: pretend the device holds `blocks` blocks per compute unit
+ *     (-1: ask the device). */
+int tt_conv2d_last_wgrad_launch(int* plan4);
+int tt_conv2d_wgrad_force_occupancy(int blocks);
 
 /* out[K] = sum over n and the HW plane of t[N,K,HW]: the bias gradient gd0.sum((0,2,3)),
  * autograd/grad_nn.py:728, :774. */

@@ -50,6 +50,8 @@ PROTOTYPES = {
     'tt_conv2d_stream_k_force_occupancy': [_I],
     'tt_conv2d_selftest_raise_async_error': [],
     'tt_conv2d_last_launch': [POINTER(c_int)],
+    'tt_conv2d_last_wgrad_launch': [POINTER(c_int)],
+    'tt_conv2d_wgrad_force_occupancy': [_I],
     'tt_conv2d_images_per_run': [_I, ctypes.c_longlong, ctypes.c_longlong, POINTER(c_int)],
     'tt_channel_sum_f32': [_P, _P, _I, _I, _I],
     'tt_workspace_size_conv2d_fwd_f32': [POINTER(c_size_t)] + [_I] * 14,

@@ -1405,6 +1405,7 @@ int dense_cell_min_tiles() { return g_dense_cell_min_tiles >= 0 ? g_dense_cell_m
 
 namespace tt {
 int conv_release_tables() { return release_tables(); }
+int conv_async_error_word(unsigned** device_pointer) { return sk_error_word(device_pointer); }
 
 // After a stream sync: has a stream-K block given up waiting for another block's partial sums since
 // the last check?  The convolution results since then are invalid in that case.
@@ -1412,7 +1413,7 @@ int conv_check_async_error() {
   if (g_sk_error_host == nullptr || *g_sk_error_host == 0u) return 0;
   *g_sk_error_host = 0u;   // the stream has drained: no kernel that could set it is running
   return tt::fail(-1, "a convolution launch timed out waiting for another block's partial sums (the device could not "
-                      "hold its grid of two blocks per compute unit); convolution results since the last "
+                      "hold its grid of resident blocks); convolution results since the last "
                       "synchronisation are invalid");
 }
 }  // namespace tt

@@ -4,8 +4,12 @@
 // m = (n, p, q) running over all N*P*Q output pixels (the reduction).  The output is small and
 // the reduction long (up to ~8e5), so the reduction is split over blockIdx.z into `splits`
 // contiguous ranges of 32-pixel chunks; each split writes an fp32 partial tile to the
-// workspace and a second kernel adds the partials in a fixed order in float64
-// (deterministic, and more accurate than one long fp32 accumulation).
+// workspace and the partials are added in a fixed order in float64 (deterministic, and more
+// accurate than one long fp32 accumulation).  When the whole grid is resident at once -- one round
+// of two blocks per compute unit, which is what the split count aims for -- the adding happens
+// inside the kernel: every block publishes its partial tile (write-through stores, then a flag),
+// waits for the flags of the other splits of its tile, and adds 1/splits of the tile's elements
+// over all splits.  Otherwise a second kernel (wgrad_reduce) adds them.
 //
 // Both operands are contiguous along the reduction index in NCHW memory, so lanes run along
 // pixels for coalesced loads and the LDS tiles are [row][pixel] with a 4-float pad: an MFMA
@@ -59,11 +63,34 @@ struct Wgrad {
   // entries from M to chunks*32 hold {N-1, bit 31, 0, all ones}.  Built once per geometry.
   const int4* pixtab;
   const int* pixhi;   // kernels of 32 .. 63 taps: bits 32 .. 63 of every pixel's tap mask
+  // partial sums added inside the kernel (fuse != 0; the grid is one round of resident blocks):
+  // `out` is dw itself, partial tiles go to fusePartial[group * tiles + tile][split] in the
+  // accumulators' own register order, 16 bytes per lane
+  int fuse;
+  floatx4* fusePartial;
+  unsigned* fuseFlags;    // [(group * tiles + tile) * splits + split] = fuseEpoch once the partial is in memory
+  unsigned fuseEpoch;     // differs from launch to launch: the flags never need clearing
+  unsigned* fuseError;    // pinned host word, set when a wait for a flag ran out
+  int fuseKL, fuseNf;     // lanes along the splits, and float4s per pass, of the adding stage (KL * Nf = 256)
 };
 
 constexpr int kSrdFlags = 0x00020000;     // raw buffer, 32-bit data format
 constexpr int kSrdRecords = 0x7fffffff;   // offsets with bit 31 set are out of range and read 0
 __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
+
+// 16-byte buffer accesses at system scope (cache-policy bits sc0 | sc1): written through to memory,
+// read from memory, past the per-XCD L2s, which do not snoop each other.  Partial tiles travel
+// between blocks on different XCDs this way; ordering is by completion (the writer waits for its
+// stores before its flag goes up, the reader loads after it has seen the flag).
+constexpr int kSystemScope = 1 | 16;
+constexpr int kFuseFlagWords = 4096, kFuseSpinLimit = 1 << 22;
+__device__ __forceinline__ void store_coherent(__amdgpu_buffer_rsrc_t rsrc, int byte_off, floatx4 v) {
+  typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, v), rsrc, byte_off, 0, kSystemScope);
+}
+__device__ __forceinline__ floatx4 load_coherent(__amdgpu_buffer_rsrc_t rsrc, int byte_off) {
+  return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, kSystemScope));
+}
 
 // Two blocks per CU is all the LDS tiles allow: tell the compiler not to squeeze registers (and
 // spill) for a third wave per SIMD.
@@ -382,6 +409,90 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     if (c < c_end) chunk_body(0, last, last);
   }
 
+  if (p.fuse) {
+    // ---- partial sums added inside the kernel --------------------------------------------------
+    // Publish: the accumulators as they lie in registers, one coalesced 16-byte store per lane and
+    // quad, written through to memory; every wave waits for its stores, then one thread raises the
+    // block's flag to this launch's epoch.
+    constexpr int F4 = MT * NT * 4 * kThreads;   // float4s of one tile
+    const int S = (int)gridDim.z;
+    const int tl = g * (int)gridDim.x + tile;
+    const __amdgpu_buffer_rsrc_t part =
+        __builtin_amdgcn_make_buffer_rsrc((void*)(p.fusePartial + (size_t)tl * S * F4), 0, kSrdRecords, kSrdFlags);
+#pragma unroll
+    for (int xx = 0; xx < MT; ++xx)
+#pragma unroll
+      for (int yy = 0; yy < NT; ++yy)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          store_coherent(part, 16 * (split * F4 + ((xx * NT + yy) * 4 + q) * kThreads + tid),
+                         floatx4{acc[xx][yy][4 * q], acc[xx][yy][4 * q + 1], acc[xx][yy][4 * q + 2], acc[xx][yy][4 * q + 3]});
+    __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0)
+    __syncthreads();
+    unsigned* flags = p.fuseFlags + (size_t)tl * S;
+    if (tid == 0) __hip_atomic_store(&flags[split], p.fuseEpoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    // Wait for every split of this tile (all blocks of the grid are resident and publish as soon as
+    // their reduction range is done, so nobody waits on somebody who waits).  Bounded all the same:
+    // a wait that runs out raises the error word that the host reports at its next synchronisation.
+    for (int j = tid; j < S; j += kThreads) {
+      int spins = 0;
+      while (__hip_atomic_load(&flags[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != p.fuseEpoch) {
+        if (++spins >= kFuseSpinLimit) {
+          __hip_atomic_store(p.fuseError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+    }
+    __syncthreads();
+    // Add: this block owns float4s [split * nf, (split + 1) * nf) of the tile, nf = ceil(F4 / S).
+    // Thread (kl, fi) adds splits kl, kl + KL, ... of float4 fi in float64; the KL sums of a float4
+    // are then added in kl order.  The order is fixed by the geometry alone: results are
+    // bit-reproducible.
+    const int nf = (F4 + S - 1) / S;
+    const int lo = split * nf, hi = min(F4, lo + nf);
+    const int KL = p.fuseKL, NF = p.fuseNf;
+    const int fi = tid % NF, kl = tid / NF;
+    double* comb = reinterpret_cast<double*>(&As[0][0][0]);   // [KL][NF][4]; the tiles are no longer read
+    float* __restrict__ dwg = p.out + (size_t)g * p.Kg * p.J;
+    for (int base = lo; base < hi; base += NF) {
+      const int f = base + fi;
+      double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+      if (f < hi) {
+#pragma unroll 4
+        for (int k = kl; k < S; k += KL) {
+          const floatx4 v = load_coherent(part, 16 * (k * F4 + f));
+          s0 += (double)v[0]; s1 += (double)v[1]; s2 += (double)v[2]; s3 += (double)v[3];
+        }
+      }
+      if (kl > 0) {
+        double* c = comb + ((size_t)kl * NF + fi) * 4;
+        c[0] = s0; c[1] = s1; c[2] = s2; c[3] = s3;
+      }
+      __syncthreads();
+      if (kl == 0 && f < hi) {
+        for (int l = 1; l < KL; ++l) {
+          const double* c = comb + ((size_t)l * NF + fi) * 4;
+          s0 += c[0]; s1 += c[1]; s2 += c[2]; s3 += c[3];
+        }
+        // float4 f of the tile = accumulator quad (xx, yy, q) of thread t: rows 8q + 4h .. +3, one column
+        const int t = f % kThreads, idx = f / kThreads;
+        const int q = idx & 3, yy = (idx >> 2) % NT, xx = (idx >> 2) / NT;
+        const int tw = t >> 6, tl32 = t & 31, th = (t >> 5) & 1;
+        const int i = i0 + ((tw / WN) * MT + xx) * 32 + 8 * q + 4 * th;
+        const int j = j0 + ((tw % WN) * NT + yy) * 32 + tl32;
+        if (j < p.J) {
+          if (i < p.Kg) dwg[(size_t)i * p.J + j] = (float)s0;
+          if (i + 1 < p.Kg) dwg[(size_t)(i + 1) * p.J + j] = (float)s1;
+          if (i + 2 < p.Kg) dwg[(size_t)(i + 2) * p.J + j] = (float)s2;
+          if (i + 3 < p.Kg) dwg[(size_t)(i + 3) * p.J + j] = (float)s3;
+        }
+      }
+      __syncthreads();
+    }
+    return;
+  }
+
   float* __restrict__ out = p.out + (size_t)split * p.outStrideSplit + (size_t)g * p.Kg * p.J;
 #pragma unroll
   for (int yy = 0; yy < NT; ++yy) {
@@ -667,28 +778,59 @@ int cached_pixtab(const char* fn, const PixGeom& g, bool wide, bool host_only, c
   return 0;
 }
 
+typedef void (*WgradKernel)(const Wgrad);
 template <int WM, int WN, int MT, int NT>
-void launch_wgrad(const Wgrad& p, dim3 grid, bool buf, bool va, bool vb, bool wide, hipStream_t st) {
+WgradKernel pick_wgrad(bool buf, bool va, bool vb, bool wide) {
   if (wide) {   // implies buf and not vb
     const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
-    if (bf && va) wgrad_wide_bf16<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
-    else if (bf) wgrad_wide_bf16<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
-    else if (va) wgrad_wide_f32<WM, WN, MT, NT, true><<<grid, kThreads, 0, st>>>(p);
-    else wgrad_wide_f32<WM, WN, MT, NT, false><<<grid, kThreads, 0, st>>>(p);
-    return;
+    if (bf && va) return wgrad_wide_bf16<WM, WN, MT, NT, true>;
+    if (bf) return wgrad_wide_bf16<WM, WN, MT, NT, false>;
+    if (va) return wgrad_wide_f32<WM, WN, MT, NT, true>;
+    return wgrad_wide_f32<WM, WN, MT, NT, false>;
   }
   if (tt::conv_math() == TT_CONV_MATH_BF16) {
-    if (buf && va && vb) wgrad_bf16<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
-    else if (buf && va) wgrad_bf16<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
-    else if (buf) wgrad_bf16<WM, WN, MT, NT, true, false, false><<<grid, kThreads, 0, st>>>(p);
-    else wgrad_bf16<WM, WN, MT, NT, false, false, false><<<grid, kThreads, 0, st>>>(p);
-    return;
+    if (buf && va && vb) return wgrad_bf16<WM, WN, MT, NT, true, true, true>;
+    if (buf && va) return wgrad_bf16<WM, WN, MT, NT, true, true, false>;
+    if (buf) return wgrad_bf16<WM, WN, MT, NT, true, false, false>;
+    return wgrad_bf16<WM, WN, MT, NT, false, false, false>;
   }
-  if (buf && va && vb) wgrad_f32<WM, WN, MT, NT, true, true, true><<<grid, kThreads, 0, st>>>(p);
-  else if (buf && va) wgrad_f32<WM, WN, MT, NT, true, true, false><<<grid, kThreads, 0, st>>>(p);
-  else if (buf) wgrad_f32<WM, WN, MT, NT, true, false, false><<<grid, kThreads, 0, st>>>(p);
-  else wgrad_f32<WM, WN, MT, NT, false, false, false><<<grid, kThreads, 0, st>>>(p);
+  if (buf && va && vb) return wgrad_f32<WM, WN, MT, NT, true, true, true>;
+  if (buf && va) return wgrad_f32<WM, WN, MT, NT, true, true, false>;
+  if (buf) return wgrad_f32<WM, WN, MT, NT, true, false, false>;
+  return wgrad_f32<WM, WN, MT, NT, false, false, false>;
 }
+
+// Blocks of `kernel` that the device holds at once (asked once per kernel: registers and LDS of the
+// compiled code decide it).  The in-kernel adding of the partial sums is used only for grids that
+// fit: all blocks of a tile wait for each other.
+int g_wgrad_forced_occupancy = -1;   // >= 0: pretend this many blocks per compute unit (tests of the fallback)
+long long resident_blocks(WgradKernel kernel) {
+  static std::map<WgradKernel, int> cache;
+  auto it = cache.find(kernel);
+  if (it == cache.end()) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, kThreads, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      n = 0;
+    }
+    it = cache.emplace(kernel, n).first;
+  }
+  const int per_cu = g_wgrad_forced_occupancy >= 0 ? g_wgrad_forced_occupancy : it->second;
+  return (long long)per_cu * tt::compute_units();
+}
+
+unsigned g_fuse_epoch = 0;
+unsigned* g_fuse_flags = nullptr;
+int fuse_flags(unsigned** out) {
+  if (g_fuse_flags == nullptr) {
+    const size_t bytes = sizeof(unsigned) * kFuseFlagWords;
+    TT_HIP(hipMalloc((void**)&g_fuse_flags, bytes));
+    TT_HIP(hipMemsetAsync(g_fuse_flags, 0, bytes, tt::stream()));
+  }
+  *out = g_fuse_flags;
+  return 0;
+}
+int g_last_wgrad[4] = {};   // instrumentation: {tiles * groups, splits, partial sums added in the kernel, slots}
 
 }  // namespace
 
@@ -777,22 +919,24 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
   }
 
   const size_t elems = (size_t)groups * Kg * J;
+  // Partial sums added inside the kernel: one run, several splits, and every partial tile of the
+  // grid (padded to whole tiles, 16 bytes per lane) addressable with 32-bit byte offsets per tile.
+  const size_t fuse_bytes = sizeof(float) * (size_t)bm * bn * (size_t)tiles * (size_t)slots;
+  const bool fuse_shape = runs.size() == 1 && slots > 1 && tiles * slots <= kFuseFlagWords &&
+                          (long long)slots * bm * bn * 4 < (1LL << 31);
   if (size_only) {
-    *size_only = slots > 1 ? sizeof(float) * elems * slots : 0;
+    const size_t plain = slots > 1 ? sizeof(float) * elems * slots : 0;
+    *size_only = fuse_shape && fuse_bytes > plain ? fuse_bytes : plain;
     return 0;
   }
-  float* target = dw;
-  if (slots > 1 && !check_only) {
-    void* ws;
-    if (tt::workspace(sizeof(float) * elems * slots, &ws)) return -1;
-    target = (float*)ws;
-  }
   hipStream_t st = check_only ? nullptr : tt::stream();
+  float* target = dw;
+  void* ws = nullptr;
+  bool fused = false;
   for (const Run& r : runs) {
     Wgrad p{};
     p.x = x + (size_t)r.n0 * C * H * W;
     p.dy = dy + (size_t)r.n0 * K * P * Q;
-    p.out = target + (size_t)r.slot0 * elems;
     p.Kg = Kg; p.J = J; p.M = r.n * P * Q;
     p.chunks = r.chunks; p.chunksPerSplit = r.cps;
     p.divPQ = tt::make_fastdiv((uint32_t)(P * Q));
@@ -822,26 +966,65 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
     const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)p.dy & 15) == 0;
     const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)p.x & 15) == 0;
+    WgradKernel kernel;
+    if (bm == 128 && bn == 128) kernel = pick_wgrad<2, 2, 2, 2>(buf, va, vb, wide);
+    else if (bm == 64 && bn == 128) kernel = pick_wgrad<2, 2, 1, 2>(buf, va, vb, wide);
+    else if (bm == 128 && bn == 64) kernel = pick_wgrad<2, 2, 2, 1>(buf, va, vb, wide);
+    else kernel = pick_wgrad<2, 2, 1, 1>(buf, va, vb, wide);
+    if (ws == nullptr && slots > 1) {   // first run: now the kernel is known, and with it what the device holds of it
+      fused = fuse_shape && tiles * r.splits <= resident_blocks(kernel);
+      if (tt::workspace(fused ? fuse_bytes : sizeof(float) * elems * slots, &ws)) return -1;
+      target = (float*)ws;
+    }
+    p.out = target + (size_t)r.slot0 * elems;
+    if (fused) {
+      p.out = dw;
+      p.fuse = 1;
+      p.fusePartial = (floatx4*)ws;
+      if (fuse_flags(&p.fuseFlags) || tt::conv_async_error_word(&p.fuseError)) return -1;
+      if (++g_fuse_epoch == 0) ++g_fuse_epoch;
+      p.fuseEpoch = g_fuse_epoch;
+      // adding stage: nf float4s per block; KL lanes along the splits for each, KL * NF = 256
+      const int nf = ceil_div((long long)bm * bn / 4, r.splits);
+      int KL = 1;
+      while (KL < 32 && 2 * KL * nf <= kThreads && 2 * KL <= r.splits) KL *= 2;
+      p.fuseKL = KL;
+      p.fuseNf = kThreads / KL;
+    }
+    const int plan[4] = {(int)tiles, r.splits, fused ? 1 : 0, slots};
+    std::copy(plan, plan + 4, g_last_wgrad);
     dim3 grid(tilesI * tilesJ, groups, r.splits);
     {
       tt::ProfScope prof(TT_PROF_CONV_WGRAD);
-      if (bm == 128 && bn == 128)
-        launch_wgrad<2, 2, 2, 2>(p, grid, buf, va, vb, wide, st);
-      else if (bm == 64 && bn == 128)
-        launch_wgrad<2, 2, 1, 2>(p, grid, buf, va, vb, wide, st);
-      else if (bm == 128 && bn == 64)
-        launch_wgrad<2, 2, 2, 1>(p, grid, buf, va, vb, wide, st);
-      else
-        launch_wgrad<2, 2, 1, 1>(p, grid, buf, va, vb, wide, st);
+      hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, st, p);
     }
     TT_LAUNCH_CHECK();
   }
   if (check_only) return 0;
-  if (slots > 1) {
+  if (slots > 1 && !fused) {
     tt::ProfScope prof(TT_PROF_CONV_WGRAD_REDUCE);
     wgrad_reduce<<<ceil_div((long long)elems, 256), kThreads, 0, st>>>(target, dw, elems, slots);
     TT_LAUNCH_CHECK();
   }
+  return 0;
+}
+
+// Instrumentation (tests): {tiles, reduction splits, 1 if the partial sums were added inside the
+// kernel, partial-sum slots} of the last weight-gradient launch.
+int tt_conv2d_last_wgrad_launch(int* plan4) {
+  TT_API_LOCK();
+  TT_REQUIRE(plan4 != nullptr, "tt_conv2d_last_wgrad_launch: null result pointer");
+  std::copy(g_last_wgrad, g_last_wgrad + 4, plan4);
+  return 0;
+}
+
+// Instrumentation (tests): pretend the device holds `blocks` blocks of every weight-gradient kernel
+// per compute unit (-1: ask the device), so that the separate reduce kernel can be exercised on
+// shapes that would otherwise add their partial sums inside the kernel.
+int tt_conv2d_wgrad_force_occupancy(int blocks) {
+  TT_API_LOCK();
+  TT_REQUIRE(blocks >= -1 && blocks <= 64, "tt_conv2d_wgrad_force_occupancy: %d is out of range (-1..64)", blocks);
+  g_wgrad_forced_occupancy = blocks;
   return 0;
 }
 

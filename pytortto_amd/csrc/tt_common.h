@@ -44,6 +44,9 @@ int conv_release_tables();
 int wgrad_release_tables();
 // After a stream sync: reports (once) a convolution launch whose blocks gave up waiting for each other.
 int conv_check_async_error();
+// Device pointer of the one word (pinned host memory) that such a block sets; shared by the
+// forward / input-gradient kernels and the weight gradient.
+int conv_async_error_word(unsigned** device_pointer);
 
 // Brackets the launches made during its lifetime with events when profiling is enabled
 // (a negative kernel id switches it off for that scope).

@@ -341,3 +341,87 @@ def test_stream_k_partial_sums_across_many_launches():
         np.testing.assert_allclose(first, y_ref, rtol=1e-4, atol=1e-5)
         for y in ys[1:]:
             np.testing.assert_array_equal(y.get(), first)
+
+
+def _last_wgrad():
+    import ctypes
+    from pytortto_amd import _hip
+    plan = (ctypes.c_int * 4)()
+    _hip.call('tt_conv2d_last_wgrad_launch', plan)
+    return dict(zip(('tiles', 'splits', 'added_in_kernel', 'slots'), plan))
+
+
+# weight gradients whose partial sums are added inside the kernel (one round of resident blocks):
+# ragged rows and columns, 1x1 / 3x3 / stem taps, groups, one tile with hundreds of splits, many tiles with few
+WGRAD_FUSED_CASES = [
+    (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # 64x64 tiles, J = 576: nine tiles, 56 splits each
+    (16, 64, 56, 56, 64, 1, 1, (1, 1), (0, 0), (1, 1), 1),       # one 64x64 tile, hundreds of splits: two float4s per block
+    (8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1),         # stem: J = 147 in three 64-column tiles, 64-bit tap masks
+    (3, 96, 15, 15, 200, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # ragged rows (200) and columns (864)
+    (8, 256, 14, 14, 512, 1, 1, (1, 1), (0, 0), (1, 1), 1),      # 128x64 tiles, 16 tiles
+    (4, 64, 20, 20, 96, 3, 3, (1, 1), (2, 2), (2, 2), 4),        # groups: tiles of every group share the grid
+    (32, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # 36 tiles of 128x128, 14 splits
+    (6, 20, 9, 9, 36, 3, 3, (1, 1), (1, 1), (1, 1), 1),          # J = 180, rows 36: small ragged tiles
+]
+
+
+@pytest.mark.parametrize('case', WGRAD_FUSED_CASES)
+def test_weight_gradient_with_partial_sums_added_in_the_kernel(case):
+    """dw against the oracle and float64 with the in-kernel adding, the same bits on a second call, and
+    the same values (to float64-sum rounding) from the separate reduce kernel, which the library takes
+    when the device would not hold the whole grid (forced here)."""
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((n, c, h, w_)).astype(np.float32)
+    p = (h + 2 * pd[0] - dl[0] * (r - 1) - 1) // st[0] + 1
+    q = (w_ + 2 * pd[1] - dl[1] * (s - 1) - 1) // st[1] + 1
+    gy = rng.standard_normal((n, k, p, q)).astype(np.float32)
+    w_shape = (k, c // g, r, s)
+    zero_w = np.zeros(w_shape, np.float32)
+    _, xpad = oracle.convolution_forward(x, zero_w, None, st, pd, dl, g)
+    _, dw32, _ = oracle.convolution_backward(gy, x, xpad, zero_w, st, pd, dl, g, need=(False, True, False))
+    _, xpad64 = oracle.convolution_forward(x.astype(np.float64), zero_w.astype(np.float64), None, st, pd, dl, g)
+    _, dw64, _ = oracle.convolution_backward(gy.astype(np.float64), x.astype(np.float64), xpad64, zero_w.astype(np.float64),
+                                             st, pd, dl, g, need=(False, True, False))
+    xd, gyd = hiparray(x), hiparray(gy)
+    dw = ops.conv2d_wgrad(xd, gyd, w_shape, st, pd, dl, g).get()
+    plan = _last_wgrad()
+    assert plan['added_in_kernel'] == 1 and plan['splits'] > 1, plan
+    _check('dw', dw, dw32, dw64, reduction=True)
+    ops.conv2d_fwd(xd, hiparray(rng.standard_normal(w_shape).astype(np.float32)), None, st, pd, dl, g)   # other work in between
+    np.testing.assert_array_equal(ops.conv2d_wgrad(xd, gyd, w_shape, st, pd, dl, g).get(), dw)
+    _hip.call('tt_conv2d_wgrad_force_occupancy', 0)
+    try:
+        dw_two_kernels = ops.conv2d_wgrad(xd, gyd, w_shape, st, pd, dl, g).get()
+        assert _last_wgrad()['added_in_kernel'] == 0
+    finally:
+        _hip.call('tt_conv2d_wgrad_force_occupancy', -1)
+    _check('dw (reduce kernel)', dw_two_kernels, dw32, dw64, reduction=True)
+    scale = float(np.abs(dw64).max())
+    np.testing.assert_allclose(dw, dw_two_kernels, rtol=0, atol=2e-7 * scale)     # both sum float32 partials in float64
+
+
+def test_weight_gradient_fused_launches_back_to_back_reuse_their_flags():
+    """Different layers one after the other re-use the same partial-sum slots and flag words; the flag
+    value changes from launch to launch, so nothing left over from the launch before can be taken for
+    this launch's: the same bits every time, and the right ones."""
+    from pytortto_amd import ops
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(22)
+    layers = []
+    for case in WGRAD_FUSED_CASES[:5]:
+        n, c, h, w_, k, r, s, st, pd, dl, g = case
+        p = (h + 2 * pd[0] - dl[0] * (r - 1) - 1) // st[0] + 1
+        q = (w_ + 2 * pd[1] - dl[1] * (s - 1) - 1) // st[1] + 1
+        layers.append((hiparray(rng.standard_normal((n, c, h, w_)).astype(np.float32)),
+                       hiparray(rng.standard_normal((n, k, p, q)).astype(np.float32)), (k, c // g, r, s), (st, pd, dl, g)))
+    first = None
+    for _ in range(6):
+        outs = [ops.conv2d_wgrad(x, gy, shape, *geo) for x, gy, shape, geo in layers]
+        got = [o.get() for o in outs]
+        if first is None:
+            first = got
+        for a, b in zip(first, got):
+            np.testing.assert_array_equal(a, b)
