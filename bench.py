@@ -694,9 +694,11 @@ def main():
                      'achieved': round(bf_igemm_tflops, 2), 'peak': PEAK_BF16_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(bf_igemm_tflops / PEAK_BF16_MFMA_TFLOPS, 4), 'traffic': None,
                      'speedup_over_f32_kernel': round((ms_fwd + ms_dg) / bf_igemm_ms, 2),
-                     'note': 'tensors stay fp32 in HBM and the gathered operand is fetched one 4-byte element per lane: the '
-                             'fetch path (address unit busy 50-70 % of cycles) and one barrier per 16-deep chunk bound the '
-                             'kernel, not the matrix pipe'},
+                     'note': 'tensors stay fp32 in HBM.  Forward and stride-1 input gradients run on bf16-first kernels '
+                             '(operands converted on their way into LDS, 32-deep chunks): their 1x1 layers move their bytes at '
+                             'HBM speed, their 3x3 layers are bound by the address unit (one 4-byte gathered element per lane); '
+                             'launches with fewer tiles than compute units and long reductions, strided input gradients and the '
+                             'stem stay on the float32 kernels\' bf16 instantiations'},
         'wgrad_tflops': round(flops_per_pass * args.steps / (bf_prof['conv_wgrad'][1] * 1e-3) / 1e12, 2),
         'kernels_ms_per_step': {k: round(v[1] / args.steps, 4) for k, v in bf_prof.items() if v[0]}}
     del layers

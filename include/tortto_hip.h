@@ -199,7 +199,8 @@ int tt_conv2d_selftest_raise_async_error(void);
 int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* per);
 /* The plan of the last single matrix-product launch made by tt_conv2d_fwd_f32 / _dgrad_f32 (host
  * pointer to 8 ints): tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent
- * grid (0 = one tile per block), tiles computed whole, blocks sharing the remaining tiles'
+ * grid (0 = one tile per block, -1 = one tile per block on the bf16-first kernels), tiles computed
+ * whole, blocks sharing the remaining tiles'
  * reductions, addressing mode.  Tests use it to compare the images where the shared tiles begin. */
 int tt_conv2d_last_launch(int* plan8);
 /* The same for the weight gradient, whose blocks add each other's partial sums inside the kernel
@@ -208,6 +209,14 @@ int tt_conv2d_last_launch(int* plan8);
  *     slots} of the last launch (host pointer to 4 ints);
  *   tt_conv2d_wgrad_force_occupancy: pretend the device holds `blocks` blocks per compute unit
  *     (-1: ask the device). */
+/* tt_conv2d_bf16_first_enable: with TT_CONV_MATH_BF16 selected, forward and stride-1 input-gradient
+ * launches go to kernels built around the bf16 matrix instruction (operands converted on their way
+ * into LDS, 32-deep chunks) when they have at least one tile per compute unit or a reduction of at
+ * most 1024 (1, the default) or whenever those kernels support the geometry (2: small test shapes);
+ * 0 keeps every launch on the float32 kernels' bf16 instantiations, which also serve the launches
+ * the former do not take.  Both compute the same thing: the convolution of
+ * the bf16-rounded operands in float32. */
+int tt_conv2d_bf16_first_enable(int on);
 int tt_conv2d_last_wgrad_launch(int* plan4);
 int tt_conv2d_wgrad_force_occupancy(int blocks);
 

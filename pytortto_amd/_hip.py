@@ -51,6 +51,7 @@ PROTOTYPES = {
     'tt_conv2d_selftest_raise_async_error': [],
     'tt_conv2d_last_launch': [POINTER(c_int)],
     'tt_conv2d_last_wgrad_launch': [POINTER(c_int)],
+    'tt_conv2d_bf16_first_enable': [_I],
     'tt_conv2d_wgrad_force_occupancy': [_I],
     'tt_conv2d_images_per_run': [_I, ctypes.c_longlong, ctypes.c_longlong, POINTER(c_int)],
     'tt_channel_sum_f32': [_P, _P, _I, _I, _I],

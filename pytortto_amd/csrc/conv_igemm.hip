@@ -37,82 +37,11 @@
 #include <type_traits>
 #include <vector>
 
-#include "tt_common.h"
+#include "conv_igemm_common.h"
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-
-constexpr int kThreads = 256;
-constexpr int kBKQ = 4;          // k-quads per chunk (BK = 16)
-constexpr int kInvalid = -(1 << 20);
-
-// One entry per reduction index k (padded with never-valid entries to a whole chunk).
-struct KEntry {
-  int off;   // element offset added to the pixel's base offset (tap-mask tables: byte offset, biased to be >= 0)
-  int dhw;   // (row step & 0xffff) | (column step << 16), both signed 16 bit (tap-mask tables: tap number; 31, or 63 with the 64-bit mask, = padding)
-};
-
-typedef int intx2 __attribute__((ext_vector_type(2)));
-typedef const intx2 __attribute__((address_space(4))) * ConstKTab;   // constant address space: scalar (s_load) access
-
-struct Igemm {
-  const float* src;
-  const floatx4* wp;     // [G][KQ][Ipad] x 4 floats
-  const KEntry* ktab;    // [KQ*4]
-  const float* bias;     // [G*I] or null
-  float* out;
-  int I, Ipad, KQ, M;
-  tt::FastDiv divUV, divV;   // m -> (n, u, v)
-  int su, bh, sv, bw;        // ih0 = u*su + bh, iw0 = v*sv + bw
-  int Hlim, Wlim, srcRow;
-  int srcStrideN, srcStrideG;
-  int outStrideN, outStrideG, outStrideI, outRow;
-  int ou, ouh, ov, ovw;      // output row = u*ou + ouh, column = v*ov + ovw
-  int tilesI;                // row tiles per group
-  int tiles;                 // tilesI * pixel tiles
-  // forward launches whose weight rows are a multiple of 4 long read the weights in place (a
-  // row of w is already k-major): row stride in floats, 0 = use the repacked copy in wp
-  const float* wraw;
-  int wRowStride;
-  // How the gathered operand is addressed:
-  //   kModeCompare: 64-bit addresses, bounds compared per element (any geometry, any size)
-  //   kModeGemm   : 1x1, stride 1, no padding: the operand is the [k][pixel] matrix of each image
-  //                 itself; 16-byte buffer loads along pixels, kStride elements between k rows
-  //   kModeTapMask: buffer loads; per tile every lane keeps one bit per tap (TB x TC <= 31 taps)
-  //                 telling whether that tap falls outside the image for its pixel
-  //   kModeTapMask64: the same with a 64-bit mask (32 .. 63 taps: 7x7 kernels), one 64-bit shift
-  //                 per element instead of a 32-bit one
-  // The two buffer modes address relative to the first image of the tile with 32-bit byte
-  // offsets; the host selects them only when those stay below 2 GiB.
-  int mode;
-  int kStride, Kred;
-  int TB, TC, stepH, stepW;  // tap window and steps of the table (tap-mask mode)
-  int voffBias;              // elements added to every lane offset so that it is never negative
-  long long srdBias;         // elements subtracted from the buffer base to make up for all biases
-  const void* wbuf;          // buffer modes: base of the weight operand (wp or wraw)
-  // buffer-mode input gradients of 1x1 layers read w[k][c] in place, transposed: row i of the
-  // GEMM is column c of w, so lanes (rows) are contiguous and k strides by wTransStride = C/groups
-  int wTransStride;
-  // dense input-gradient launches only (all stride-parity classes as rows of one GEMM):
-  // row i -> {element offset c*Hx*Wx + ch*Wx + cw, ch, cw, c}; output bounds outH x outW
-  const int4* rowtab;
-  int outH, outW;
-  // strided 1x1 input gradients: only one pixel of every sh x 2 cell of dx has a tap.  > 0: the
-  // launch stores each value together with the zero to its right (one 8-byte store) and zero
-  // pairs into the cellFill - 1 rows below, so dx needs no clearing beforehand
-  int cellFill;
-  // stream-K launches only: the tiles*chunks reduction steps are dealt evenly to the blocks
-  int skDpTiles;             // tiles [0, skDpTiles) are computed whole, block b takes b, b+blocks, ...
-  int skBlocks;              // blocks that share the remaining tiles' reduction steps
-  long long skIters;         // (tiles - skDpTiles) * (KQ / kBKQ)
-  floatx4* skPartial;        // [skBlocks][acc float4s per thread][256] partial accumulators, one slot per block
-  unsigned* skFlags;         // [block] = skEpoch once the block's partial is in memory
-  unsigned skEpoch;          // differs from launch to launch, so the flags never need clearing
-  unsigned* skError;         // one word in pinned host memory: set when a wait for a flag ran out
-};
+using namespace ttc;
 
 // ---- preparation kernels (tiny) --------------------------------------------------------------
 
@@ -233,11 +162,6 @@ __global__ void pack_w_dgrad_dense(const float* __restrict__ w, floatx4* __restr
 using tt::xcd_remap;
 
 typedef float floatx2 __attribute__((ext_vector_type(2)));
-constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2, kModeTapMask64 = 3;
-constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format
-constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out of range and read 0
-
-__device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cast(float, v); }
 
 // s_waitcnt vmcnt(0) in straight-line code.  Stores share the counter with loads, and the
 // compiler, unsure after a branch whether an earlier load has been waited for, repeats the wait
@@ -1108,6 +1032,10 @@ __global__ void sk_raise_error(unsigned* word) {
 
 // What the last single launch looked like (instrumentation: tests pick the images to compare from it).
 int g_last_launch[8] = {};
+// bf16 arithmetic: launches that the bf16-first kernels support go to them (tests switch this off to
+// reach the float32 kernels' bf16 instantiations on the same shapes)
+bool g_bf16_first = true;
+bool g_bf16_first_always = false;   // tests: also where the tile-count rule would keep the other kernels
 
 int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_partial) {
   tt::ProfScope prof(prof_id);
@@ -1131,10 +1059,24 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
       p.skEpoch = g_sk_epoch;
     }
   }
+  hipStream_t st = tt::stream();
+  // The reduced-precision mode's own kernels: 128-pixel tiles, one tile per block, nothing shared.
+  // They share no reduction between blocks, so launches with fewer tiles than compute units and a
+  // long reduction stay on the stream-K instantiations (measured per layer: 1.2-1.8 times faster
+  // where taken, up to 2 times slower on 100 tiles of 144 chunks).
+  const int bf_tiles = (p.Ipad / t.bm) * ceil_div(p.M, 128);
+  if (bf16_math() && g_bf16_first && bf16_first_supported(p, groups, t.bm) &&
+      ((long long)bf_tiles * groups >= cus() || p.Kred <= 1024 || g_bf16_first_always)) {
+    const int tiles = bf_tiles;
+    const int plan[8] = {t.bm, 128, tiles, p.Ipad / t.bm, -1, tiles, 0, p.mode};   // -1: the bf16-first kernels
+    std::copy(plan, plan + 8, g_last_launch);
+    bf16_first_launch(p, groups, t.bm, st);
+    TT_LAUNCH_CHECK();
+    return 0;
+  }
   const int plan[8] = {t.bm, t.bn, p.tiles, p.tilesI, t.sk_blocks, t.sk_blocks > 0 ? p.skDpTiles : p.tiles,
                        t.sk_blocks > 0 ? p.skBlocks : 0, p.mode};
   std::copy(plan, plan + 8, g_last_launch);
-  hipStream_t st = tt::stream();
   bool persistent;
   if (t.bm == 128 && t.bn == 128)
     persistent = launch_config<2, 2, 2, 2>(p, groups, t.sk_blocks, st);
@@ -1176,6 +1118,8 @@ int launch_igemm_multi(IgemmMulti& m, int groups, TileChoice t, int prof_id) {
     p.tiles = p.tilesI * ceil_div(p.M, t.bn);
     m.first[i + 1] = m.first[i] + p.tiles;
   }
+  const int plan[8] = {t.bm, t.bn, m.first[m.n], 0, 0, m.first[m.n], 0, m.c[0].mode};   // several launches in one grid
+  std::copy(plan, plan + 8, g_last_launch);
   hipStream_t st = tt::stream();
   if (t.bm == 128 && t.bn == 128)
     launch_multi_config<2, 2, 2, 2>(m, groups, st);
@@ -1438,12 +1382,21 @@ int tt_conv2d_stream_k_blocks_per_cu(int bf16, int* blocks) {
 
 // Instrumentation (tests): the plan of the last single matrix-product launch of a forward or input
 // gradient call: {tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent grid
-// (0: one tile per block), tiles computed whole (the rest share their reduction between blocks),
+// (0: one tile per block; -1: one tile per block on the bf16-first kernels), tiles computed whole (the rest share their reduction between blocks),
 // blocks sharing them, addressing mode}.  Pixel tile t starts at pixel (t / row tiles) * tile columns.
 int tt_conv2d_last_launch(int* plan8) {
   TT_API_LOCK();
   TT_REQUIRE(plan8 != nullptr, "tt_conv2d_last_launch: null result pointer");
   std::copy(g_last_launch, g_last_launch + 8, plan8);
+  return 0;
+}
+
+// Instrumentation (tests): with bf16 arithmetic selected, route the launches the bf16-first kernels
+// support to them (1, the default) or keep everything on the float32 kernels' bf16 instantiations (0).
+int tt_conv2d_bf16_first_enable(int on) {
+  TT_API_LOCK();
+  g_bf16_first = on != 0;
+  g_bf16_first_always = on == 2;   // 2: every supported launch, whatever its tile count (small test shapes)
   return 0;
 }
 

@@ -24,11 +24,15 @@ LOOSE_BOUND = 1e-2
 
 @pytest.fixture
 def bf16_math():
+    """bf16 arithmetic, with every launch the bf16-first kernels support sent to them (by default the
+    small tile counts of test shapes with long reductions would stay on the other kernels)."""
     from pytortto_amd import _hip
     _hip.set_conv_math('bf16')
+    _hip.call('tt_conv2d_bf16_first_enable', 2)
     try:
         yield
     finally:
+        _hip.call('tt_conv2d_bf16_first_enable', 1)
         _hip.set_conv_math('f32')
 
 
@@ -41,6 +45,10 @@ def _close(name, got, model, plain):
 
 @pytest.mark.parametrize('case', CONV_CASES + TILE_CASES + random_conv_cases(40, 123))
 def test_conv_bf16_forward_and_input_gradient(case, bf16_math):
+    _forward_and_input_gradient(case)
+
+
+def _forward_and_input_gradient(case):
     from pytortto_amd import ops
     from pytortto_amd.xparray import hiparray
     n, c, h, w_, k, r, s, st, pd, dl, g = case
@@ -88,6 +96,70 @@ def test_conv_transpose_bf16_forward_and_input_gradient(case, bf16_math):
     _close('y', y, y_model, y32)
     _close('dx', dx, dx_model, dx32)
     _close('dw', dw, dw_model, dw32)
+
+
+def _persistent_blocks_of_last_launch():
+    import ctypes
+    from pytortto_amd import _hip
+    plan = (ctypes.c_int * 8)()
+    _hip.call('tt_conv2d_last_launch', plan)
+    return plan[4]
+
+
+# shapes the bf16-first kernels take, one per way they fetch their operands: (forward, input gradient)
+BF16_FIRST_CASES = [
+    ((4, 64, 28, 28, 256, 1, 1, (1, 1), (0, 0), (1, 1), 1), (True, True)),      # 1x1: rows in place / columns in place, 128- and 64-row tiles
+    ((16, 256, 14, 14, 1024, 1, 1, (1, 1), (0, 0), (1, 1), 1), (True, True)),   # 1x1, 128-row tiles both ways, ragged last pixel tile
+    ((4, 64, 28, 28, 64, 1, 1, (1, 1), (0, 0), (1, 1), 1), (True, True)),       # 64-row tiles
+    ((8, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1), (True, True)),     # 3x3: tap masks, rows in place / repacked quads
+    ((16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1), (True, True)),      # 3x3 with 64-row tiles
+    ((2, 32, 12, 12, 64, 1, 1, (1, 1), (1, 1), (1, 1), 1), (True, True)),       # padded 1x1: one-tap mask, columns in place
+    ((3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2), (True, True)),         # groups
+    ((4, 128, 28, 28, 128, 3, 3, (2, 2), (1, 1), (1, 1), 1), (True, False)),    # stride 2: forward only (the input gradient's classes share a grid)
+    ((5, 32, 13, 9, 48, 5, 5, (2, 1), (4, 2), (2, 1), 2), (False, False)),      # 16 channels per group x 25 taps: not whole chunks
+    ((8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1), (False, False)),      # stem: 49 taps, dense input gradient
+]
+
+
+@pytest.mark.parametrize('case,takes', BF16_FIRST_CASES)
+def test_bf16_first_kernels_and_the_other_bf16_kernels_agree(case, takes, bf16_math):
+    """Which launches go to the bf16-first kernels, and that they and the float32 kernels' bf16
+    instantiations -- both "the convolution of the bf16-rounded operands in float32" -- agree to the
+    float32 bar on the same inputs (the summation order differs)."""
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    n, c, h, w_, k, r, s, st, pd, dl, g = case
+    rng = np.random.default_rng(8)
+    x = hiparray(rng.standard_normal((n, c, h, w_)).astype(np.float32))
+    w = hiparray((rng.standard_normal((k, c // g, r, s)) / np.sqrt(c // g * r * s)).astype(np.float32))
+    p = (h + 2 * pd[0] - dl[0] * (r - 1) - 1) // st[0] + 1
+    q = (w_ + 2 * pd[1] - dl[1] * (s - 1) - 1) // st[1] + 1
+    gy = hiparray(rng.standard_normal((n, k, p, q)).astype(np.float32))
+    y = ops.conv2d_fwd(x, w, None, st, pd, dl, g).get()
+    assert (_persistent_blocks_of_last_launch() == -1) == takes[0]
+    dx = ops.conv2d_dgrad(gy, w, None, (h, w_), st, pd, dl, g).get()
+    assert (_persistent_blocks_of_last_launch() == -1) == takes[1]
+    _hip.call('tt_conv2d_bf16_first_enable', 0)
+    try:
+        y_other = ops.conv2d_fwd(x, w, None, st, pd, dl, g).get()
+        assert _persistent_blocks_of_last_launch() != -1
+        dx_other = ops.conv2d_dgrad(gy, w, None, (h, w_), st, pd, dl, g).get()
+    finally:
+        _hip.call('tt_conv2d_bf16_first_enable', 2)
+    for name, a, b in (('y', y, y_other), ('dx', dx, dx_other)):
+        np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-5 * max(1.0, float(np.abs(b).max())), err_msg=name)
+
+
+@pytest.mark.parametrize('case', TILE_CASES)
+def test_conv_bf16_on_the_float32_kernels_instantiations(case, bf16_math):
+    """The same pins as above with the bf16-first kernels switched off: the instantiations that serve
+    whatever those do not take stay covered on every tile shape."""
+    from pytortto_amd import _hip
+    _hip.call('tt_conv2d_bf16_first_enable', 0)
+    try:
+        _forward_and_input_gradient(case)
+    finally:
+        _hip.call('tt_conv2d_bf16_first_enable', 2)
 
 
 def test_other_ops_do_not_depend_on_the_mode_and_it_switches_back():
