@@ -92,6 +92,19 @@ __device__ __forceinline__ floatx4 load_coherent(__amdgpu_buffer_rsrc_t rsrc, in
   return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, kSystemScope));
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack2(float lo, float hi) {   // two floats -> two bf16 (nearest even), lo in the low half
+  const bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(unsigned, v);
+}
+__device__ __forceinline__ int pos16(int i) { return i + (i >> 4); }   // unit of row i in a bf16 LDS line
+// The value the next lane holds (lanes 0, 2 of every quad get lanes 1, 3; odd lanes get their own).
+__device__ __forceinline__ float next_lane(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xF5 /* quad_perm [1,1,3,3] */, 0xf, 0xf, false));
+}
+
 // Two blocks per CU is all the LDS tiles allow: tell the compiler not to squeeze registers (and
 // spill) for a third wave per SIMD.
 // VA / VB (buffer path only): dy / x are fetched as 16-byte vectors of four consecutive pixels
@@ -108,8 +121,21 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   using TapBits = std::conditional_t<WIDE, uint64_t, uint32_t>;
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   constexpr int A_ROWS = VA ? BM / 32 : BM / 8, B_ROWS = VB ? BN / 32 : BN / 8;   // fetches per thread and chunk
-  __shared__ __attribute__((aligned(16))) float As[2][BM][kLd];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BN][kLd];
+  // float32 arithmetic: [row][32 pixels + pad] floats.  bf16 arithmetic: operands are rounded on their
+  // way INTO LDS and lie as 16-byte units of eight consecutive pixels of one row, [pixel / 8][row][8
+  // bf16] (one ds_read_b128 is a lane's operand of a 16-deep MFMA step; rows padded by one unit per
+  // sixteen, lines 12 or 4 units past a multiple of sixteen so that the four lines of a chunk spread
+  // over the banks): half the LDS bytes and no conversion next to the matrix instructions.
+  constexpr int ALINE = BM == 128 ? 140 : 68, BLINE = BN == 128 ? 140 : 68;
+  constexpr size_t kBytesA = BF ? sizeof(uintx4) * 2 * 4 * ALINE : sizeof(float) * 2 * BM * kLd;
+  constexpr size_t kBytesB = BF ? sizeof(uintx4) * 2 * 4 * BLINE : sizeof(float) * 2 * BN * kLd;
+  __shared__ __attribute__((aligned(16))) char lds[kBytesA + kBytesB];
+  char* const ldsA = lds;
+  char* const ldsB = lds + kBytesA;
+  float (*As)[BM][kLd] = reinterpret_cast<float (*)[BM][kLd]>(ldsA);
+  float (*Bs)[BN][kLd] = reinterpret_cast<float (*)[BN][kLd]>(ldsB);
+  uintx4 (*As16)[4][ALINE] = reinterpret_cast<uintx4 (*)[4][ALINE]>(ldsA);
+  uintx4 (*Bs16)[4][BLINE] = reinterpret_cast<uintx4 (*)[4][BLINE]>(ldsB);
   // per column j: {x offset c*HW + r*dh*W + s*dw, (r*dh) | (s*dw) << 16}; buffer path: {4 * offset, tap r*S + s}
   __shared__ int2 jtab[BN];
 
@@ -153,9 +179,12 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   const float* __restrict__ xg = p.x + (size_t)g * p.xStrideG;
 
   // staging registers of the chunk being fetched, and what its loads need
-  float areg[A_ROWS], breg[B_ROWS];
-  int amask = 0;        // all ones if this thread's pixel is inside the reduction range
-  uint32_t bok = 0;     // bit t: breg[t] is inside the image (applied when written to LDS)
+  // (bf16 arithmetic keeps two sets: the loads of the chunk after next are issued while the next
+  // chunk's values still wait in the other set for their turn to be written to LDS)
+  constexpr int SETS = BF ? 2 : 1;
+  float areg[SETS][A_ROWS], breg[SETS][B_ROWS];
+  int amask[SETS] = {};        // all ones if this thread's pixel is inside the reduction range
+  uint32_t bok[SETS] = {};     // bit t: breg[set][t] is inside the image (applied when written to LDS)
   int2 jreg[B_ROWS];
   int ih0 = kInvalid, iw0 = 0, xbase = 0, dybase = 0, alim = 0;
   const int arow = i0 + rg;
@@ -178,7 +207,7 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   }
   // vector fetches: offsets of the quad's first pixel, staging vectors, per-row x offsets
   uint32_t qvoff = 0x80000000u, qxvoff = 0x80000000u;
-  floatx4 aregv[VA ? A_ROWS : 1], bregv[VB ? B_ROWS : 1];
+  floatx4 aregv[SETS][VA ? A_ROWS : 1], bregv[SETS][VB ? B_ROWS : 1];
   int boffv[VB ? B_ROWS : 1];
   if constexpr (VB) {
 #pragma unroll
@@ -195,7 +224,7 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     if constexpr (WIDE) pixnexthi = p.pixhi[chunk * kBK + px];
     if constexpr (VA || VB) pixnextq = *reinterpret_cast<const int2*>(&p.pixtab[chunk * kBK + 4 * qpx]);
   };
-  auto decompose = [&](int chunk, int following) __attribute__((always_inline)) {
+  auto decompose = [&](int chunk, int following, const int set = 0) __attribute__((always_inline)) {
     if constexpr (BUF) {
       const int4 e = pixnext;   // entry of `chunk`
       const int2 eq = pixnextq;
@@ -227,25 +256,25 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     iw0 = (int)qq * p.sw - p.pw;
     xbase = (int)n * p.xStrideN + ((int)pp * p.sh - p.ph) * p.W + iw0;
     dybase = (int)n * p.dyStrideN + (int)pq + arow * p.PQ;
-    amask = mok ? -1 : 0;
+    amask[set] = mok ? -1 : 0;
     alim = mok ? p.Kg : 0;   // rows at or beyond it are not read (they are never stored either)
-    bok = 0;
+    bok[set] = 0;
   };
-  auto load_step = [&](int li) __attribute__((always_inline)) {
+  auto load_step = [&](int li, const int set = 0) __attribute__((always_inline)) {
     if constexpr (BUF) {
       if (li < A_ROWS) {
         if constexpr (VA)
-          aregv[li] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(dySrd, (int)(qvoff + (uint32_t)aoff[li]), 0, 0));
+          aregv[set][li] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(dySrd, (int)(qvoff + (uint32_t)aoff[li]), 0, 0));
         else
-          areg[li] = as_float(__builtin_amdgcn_raw_buffer_load_b32(dySrd, (int)(dyvoff + (uint32_t)aoff[li]), 0, 0));
+          areg[set][li] = as_float(__builtin_amdgcn_raw_buffer_load_b32(dySrd, (int)(dyvoff + (uint32_t)aoff[li]), 0, 0));
       } else {
         const int t = li - A_ROWS;
         if constexpr (VB) {
-          bregv[t] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(xSrd, (int)(qxvoff + (uint32_t)boffv[t]), 0, 0));
+          bregv[set][t] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(xSrd, (int)(qxvoff + (uint32_t)boffv[t]), 0, 0));
         } else {
           const int2 e = jreg[t];
           const uint32_t vo = ((uint32_t)(nmask >> e.y) << 31) | (xvoff + (uint32_t)e.x);
-          breg[t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
+          breg[set][t] = as_float(__builtin_amdgcn_raw_buffer_load_b32(xSrd, (int)vo, 0, 0));
         }
       }
       return;
@@ -253,37 +282,68 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     if (li < A_ROWS) {
       const int t = li;
       const bool ok = arow + 8 * t < alim;
-      areg[t] = dyg[ok ? (uint32_t)(dybase + 8 * t * p.PQ) : 0u];
+      areg[set][t] = dyg[ok ? (uint32_t)(dybase + 8 * t * p.PQ) : 0u];
     } else {
       const int t = li - A_ROWS;
       const int2 e = jreg[t];
       const int ih = ih0 + (int)(short)(e.y & 0xffff);
       const int iw = iw0 + (e.y >> 16);
       const bool ok = (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-      breg[t] = xg[ok ? (uint32_t)(xbase + e.x) : 0u];
-      bok |= ok ? (1u << t) : 0u;
+      breg[set][t] = xg[ok ? (uint32_t)(xbase + e.x) : 0u];
+      bok[set] |= ok ? (1u << t) : 0u;
     }
   };
   // Rows beyond Kg / columns beyond J may hold anything (never stored); pixels beyond M and taps
   // outside the image must be exactly zero: AND with an all-ones / all-zeros word.
-  auto store_step = [&](int buf, int li) __attribute__((always_inline)) {
-    if constexpr (BUF) {   // padding and pixels past the end were read as zeros
+  auto store_step = [&](int buf, int li, const int set = 0) __attribute__((always_inline)) {
+    if constexpr (BF) {
+      // Round to bf16 and write pixel-major units.  Vector fetches hold four consecutive pixels of a
+      // row: 8 bytes, half a unit.  Scalar fetches hold one pixel per lane: every even lane takes its
+      // neighbour's value too and writes the pair.  (Masks of the compare path apply first.)
       if (li < A_ROWS) {
-        if constexpr (VA) *reinterpret_cast<floatx4*>(&As[buf][rgq + 32 * li][4 * qpx]) = aregv[li];
-        else As[buf][rg + 8 * li][px] = areg[li];
+        if constexpr (VA) {
+          const floatx4 v = aregv[set][li];
+          *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&As16[buf][qpx >> 1][pos16(rgq + 32 * li)]) + 8 * (qpx & 1)) =
+              uintx2{pack2(v[0], v[1]), pack2(v[2], v[3])};
+        } else {
+          const float v = BUF ? areg[set][li] : __int_as_float(__float_as_int(areg[set][li]) & amask[set]);
+          const unsigned pair = pack2(v, next_lane(v));
+          if ((px & 1) == 0)
+            *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&As16[buf][px >> 3][pos16(rg + 8 * li)]) + 2 * (px & 7)) = pair;
+        }
       } else {
         const int t = li - A_ROWS;
-        if constexpr (VB) *reinterpret_cast<floatx4*>(&Bs[buf][rgq + 32 * t][4 * qpx]) = bregv[t];
-        else Bs[buf][rg + 8 * t][px] = breg[t];
+        if constexpr (VB) {
+          const floatx4 v = bregv[set][t];
+          *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&Bs16[buf][qpx >> 1][pos16(rgq + 32 * t)]) + 8 * (qpx & 1)) =
+              uintx2{pack2(v[0], v[1]), pack2(v[2], v[3])};
+        } else {
+          const int bmask = ((int)(bok[set] << (31 - t))) >> 31;
+          const float v = BUF ? breg[set][t] : __int_as_float(__float_as_int(breg[set][t]) & bmask);
+          const unsigned pair = pack2(v, next_lane(v));
+          if ((px & 1) == 0)
+            *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&Bs16[buf][px >> 3][pos16(rg + 8 * t)]) + 2 * (px & 7)) = pair;
+        }
+      }
+      return;
+    }
+    if constexpr (BUF) {   // padding and pixels past the end were read as zeros
+      if (li < A_ROWS) {
+        if constexpr (VA) *reinterpret_cast<floatx4*>(&As[buf][rgq + 32 * li][4 * qpx]) = aregv[set][li];
+        else As[buf][rg + 8 * li][px] = areg[set][li];
+      } else {
+        const int t = li - A_ROWS;
+        if constexpr (VB) *reinterpret_cast<floatx4*>(&Bs[buf][rgq + 32 * t][4 * qpx]) = bregv[set][t];
+        else Bs[buf][rg + 8 * t][px] = breg[set][t];
       }
       return;
     }
     if (li < A_ROWS) {
-      As[buf][rg + 8 * li][px] = __int_as_float(__float_as_int(areg[li]) & amask);
+      As[buf][rg + 8 * li][px] = __int_as_float(__float_as_int(areg[set][li]) & amask[set]);
     } else {
       const int t = li - A_ROWS;
-      const int bmask = ((int)(bok << (31 - t))) >> 31;
-      Bs[buf][rg + 8 * t][px] = __int_as_float(__float_as_int(breg[t]) & bmask);
+      const int bmask = ((int)(bok[set] << (31 - t))) >> 31;
+      Bs[buf][rg + 8 * t][px] = __int_as_float(__float_as_int(breg[set][t]) & bmask);
     }
   };
 
@@ -320,31 +380,24 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   constexpr int SPS = (L + (kSync - kStore) - 1) / (kSync - kStore);   // LDS writes per slot
   auto chunk_body = [&](const int buf, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
     if constexpr (BF) {
-      // Two bf16 MFMAs per accumulator contract the chunk's 32 pixels (a lane's eight k values of
-      // each are pixels 16*half + 4*h .. +3 and 16*half + 8 + 4*h .. +3, the same for both
-      // operands): a sixteenth of the fp32 matrix time, nothing to weave the loads into.
-      decompose(nchunk, nnchunk);
+      // Two bf16 MFMAs per accumulator contract the chunk's 32 pixels: step t takes pixel blocks 2t
+      // (lanes 0-31) and 2t + 1 (lanes 32-63), a lane's 16 bytes being its eight pixels, the same
+      // eight for both operands.  A sixteenth of the fp32 matrix time: nothing to weave the loads
+      // into and too short to cover their latency, so this chunk issues the loads of the chunk AFTER
+      // NEXT (`nchunk`) into staging set `buf`.
+      decompose(nchunk, nnchunk, buf);
 #pragma unroll
-      for (int li = 0; li < L; ++li) load_step(li);
+      for (int li = 0; li < L; ++li) load_step(li, buf);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        if (half == 1) read_ops(0, buf, 2);
-        read_ops(1, buf, 2 * half + 1);
+      for (int t = 0; t < 2; ++t) {
         bf16x8 a[MT], b[NT];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int xx = 0; xx < MT; ++xx)
+          a[xx] = __builtin_bit_cast(bf16x8, As16[buf][2 * t + h][pos16((wm * MT + xx) * 32 + l32)]);
 #pragma unroll
-          for (int xx = 0; xx < MT; ++xx) {
-            a[xx][j] = (__bf16)opA[0][xx][j];
-            a[xx][4 + j] = (__bf16)opA[1][xx][j];
-          }
-#pragma unroll
-          for (int yy = 0; yy < NT; ++yy) {
-            b[yy][j] = (__bf16)opB[0][yy][j];
-            b[yy][4 + j] = (__bf16)opB[1][yy][j];
-          }
-        }
+        for (int yy = 0; yy < NT; ++yy)
+          b[yy] = __builtin_bit_cast(bf16x8, Bs16[buf][2 * t + h][pos16((wn * NT + yy) * 32 + l32)]);
 #pragma unroll
         for (int xx = 0; xx < MT; ++xx)
 #pragma unroll
@@ -352,10 +405,11 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
             acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[xx], b[yy], acc[xx][yy], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
+      // the chunk after this one was fetched during the previous chunk: it has had a whole chunk's
+      // time to arrive and goes to the other LDS buffer now
 #pragma unroll
-      for (int li = 0; li < L; ++li) store_step(buf ^ 1, li);
+      for (int li = 0; li < L; ++li) store_step(buf ^ 1, li, buf ^ 1);
       __syncthreads();
-      read_ops(0, buf ^ 1, 0);
       return;
     }
 #pragma unroll
@@ -398,15 +452,28 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     for (int li = 0; li < L; ++li) load_step(li);
 #pragma unroll
     for (int li = 0; li < L; ++li) store_step(0, li);
-    __syncthreads();
-    read_ops(0, 0, 0);
     // past the end the last chunk is fetched again (cache hits) instead of branching
     int c = c_begin;
-    for (; c + 1 < c_end; c += 2) {
-      chunk_body(0, c + 1, min(c + 2, last));
-      chunk_body(1, min(c + 2, last), min(c + 3, last));
+    if constexpr (BF) {
+      // two chunks ahead: the second chunk waits in staging set 1 while the loop starts
+      decompose(min(c_begin + 1, last), min(c_begin + 2, last), 1);
+#pragma unroll
+      for (int li = 0; li < L; ++li) load_step(li, 1);
+      __syncthreads();
+      for (; c + 1 < c_end; c += 2) {
+        chunk_body(0, min(c + 2, last), min(c + 3, last));
+        chunk_body(1, min(c + 3, last), min(c + 4, last));
+      }
+      if (c < c_end) chunk_body(0, last, last);
+    } else {
+      __syncthreads();
+      read_ops(0, 0, 0);
+      for (; c + 1 < c_end; c += 2) {
+        chunk_body(0, c + 1, min(c + 2, last));
+        chunk_body(1, min(c + 2, last), min(c + 3, last));
+      }
+      if (c < c_end) chunk_body(0, last, last);
     }
-    if (c < c_end) chunk_body(0, last, last);
   }
 
   if (p.fuse) {
@@ -453,7 +520,7 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
     const int lo = split * nf, hi = min(F4, lo + nf);
     const int KL = p.fuseKL, NF = p.fuseNf;
     const int fi = tid % NF, kl = tid / NF;
-    double* comb = reinterpret_cast<double*>(&As[0][0][0]);   // [KL][NF][4]; the tiles are no longer read
+    double* comb = reinterpret_cast<double*>(lds);   // [KL][NF][4] (8 KiB); the tiles are no longer read
     float* __restrict__ dwg = p.out + (size_t)g * p.Kg * p.J;
     for (int base = lo; base < hi; base += NF) {
       const int f = base + fi;

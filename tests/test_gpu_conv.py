@@ -357,7 +357,7 @@ WGRAD_FUSED_CASES = [
     (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # 64x64 tiles, J = 576: nine tiles, 56 splits each
     (16, 64, 56, 56, 64, 1, 1, (1, 1), (0, 0), (1, 1), 1),       # one 64x64 tile, hundreds of splits: two float4s per block
     (8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1),         # stem: J = 147 in three 64-column tiles, 64-bit tap masks
-    (3, 96, 15, 15, 200, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # ragged rows (200) and columns (864)
+    (24, 96, 15, 15, 200, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # ragged rows (200) and columns (864), 128x128 tiles
     (8, 256, 14, 14, 512, 1, 1, (1, 1), (0, 0), (1, 1), 1),      # 128x64 tiles, 16 tiles
     (4, 64, 20, 20, 96, 3, 3, (1, 1), (2, 2), (2, 2), 4),        # groups: tiles of every group share the grid
     (32, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1), (1, 1), 1),     # 36 tiles of 128x128, 14 splits
