@@ -672,7 +672,7 @@ def main():
     wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
     kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
     layer_rows = None if args.no_per_layer else per_layer_table(_hip, call, layers, 20)
-    c1_gpu = single_layer_config(_hip, call, rng)
+    c1_gpu = None if args.no_per_layer else single_layer_config(_hip, call, rng)   # (kept out of profiling runs)
 
     # optional reduced-precision variant, reported separately and never part of `value`: the three
     # passes on bf16 MFMA (operands rounded inside the kernels, fp32 accumulation and tensors)

@@ -106,10 +106,22 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
  * partial sums are still combined in float64); results differ from the float32 ones by about
  * 2^-8 of the operands' magnitude per term.  It applies to tt_conv2d_fwd_f32,
  * tt_conv2d_dgrad_f32 and tt_conv2d_wgrad_f32.  The setting is process-wide and applies to
- * later calls. */
+ * later calls of every caller; the *_bf16 entry points below select it per call instead. */
 enum { TT_CONV_MATH_F32 = 0, TT_CONV_MATH_BF16 = 1 };
 int tt_set_conv_math(int mode);
 int tt_get_conv_math(int* mode);   /* host pointer */
+/* The same three passes with bf16 matrix arithmetic for one call, whatever the process-wide mode is
+ * (arguments as tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 / tt_conv2d_wgrad_f32 below; tensors are
+ * float32): for callers that must not change what other callers of the library compute. */
+int tt_conv2d_fwd_bf16(const float* x, const float* w, const float* bias, float* y,
+                       int N, int C, int H, int W, int K, int R, int S,
+                       int sh, int sw, int ph, int pw, int dh, int dw, int groups);
+int tt_conv2d_dgrad_bf16(const float* dy, const float* w, const float* bias, float* dx,
+                         int N, int C, int Hx, int Wx, int K, int R, int S,
+                         int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q);
+int tt_conv2d_wgrad_bf16(const float* x, const float* dy, float* dw,
+                         int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q);
 
 /* Tuning threshold of tt_conv2d_dgrad_f32 for strided layers with very few input channels (the
  * ResNet stem, the output layer of a transposed generator), no counterpart in the reference.

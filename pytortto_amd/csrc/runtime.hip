@@ -300,6 +300,38 @@ int tt_get_conv_math(int* mode) {
   return 0;
 }
 
+// The three convolution passes with bf16 matrix arithmetic for this call only, whatever the
+// process-wide mode is: the mode is switched under the API lock, which this thread holds for the
+// whole call, so no other caller can see the switch.
+namespace {
+struct ScopedBf16 {
+  int saved;
+  ScopedBf16() : saved(S().conv_math) { S().conv_math = TT_CONV_MATH_BF16; }
+  ~ScopedBf16() { S().conv_math = saved; }
+};
+}  // namespace
+
+int tt_conv2d_fwd_bf16(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
+                       int R, int S_, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
+  TT_API_LOCK();
+  ScopedBf16 mode;
+  return tt_conv2d_fwd_f32(x, w, bias, y, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw, groups);
+}
+
+int tt_conv2d_dgrad_bf16(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
+                         int K, int R, int S_, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q) {
+  TT_API_LOCK();
+  ScopedBf16 mode;
+  return tt_conv2d_dgrad_f32(dy, w, bias, dx, N, C, Hx, Wx, K, R, S_, sh, sw, ph, pw, dh, dw, groups, P, Q);
+}
+
+int tt_conv2d_wgrad_bf16(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S_,
+                         int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+  TT_API_LOCK();
+  ScopedBf16 mode;
+  return tt_conv2d_wgrad_f32(x, dy, dw, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw_, groups, P, Q);
+}
+
 int tt_sync(void) {
   TT_REQUIRE_INIT();
   TT_HIP(hipStreamSynchronize(S().stream));

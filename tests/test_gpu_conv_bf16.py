@@ -188,6 +188,37 @@ def test_other_ops_do_not_depend_on_the_mode_and_it_switches_back():
         _hip.set_conv_math('fp8')
 
 
+def test_per_call_bf16_entry_points_leave_the_process_wide_mode_alone():
+    """tt_conv2d_*_bf16: bf16 arithmetic for one call; the same bits as the float32-named entry points
+    give under tt_set_conv_math(bf16), and the mode other callers see is float32 before and after."""
+    from pytortto_amd import _hip, ops
+    from pytortto_amd.xparray import hiparray
+    rng = np.random.default_rng(10)
+    n, c, h, k = 4, 32, 14, 48
+    x = hiparray(rng.standard_normal((n, c, h, h), dtype=np.float32))
+    w = hiparray(rng.standard_normal((k, c, 3, 3), dtype=np.float32))
+    gy = hiparray(rng.standard_normal((n, k, h, h), dtype=np.float32))
+    geo = ((1, 1), (1, 1), (1, 1), 1)
+    a = (n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1)
+    y, dx, dw = hiparray.empty((n, k, h, h)), hiparray.empty((n, c, h, h)), hiparray.empty((k, c, 3, 3))
+    assert _hip.get_conv_math() == 'f32'
+    _hip.call('tt_conv2d_fwd_bf16', x.ptr, w.ptr, None, y.ptr, *a)
+    _hip.call('tt_conv2d_dgrad_bf16', gy.ptr, w.ptr, None, dx.ptr, *a, h, h)
+    _hip.call('tt_conv2d_wgrad_bf16', x.ptr, gy.ptr, dw.ptr, *a, h, h)
+    assert _hip.get_conv_math() == 'f32'
+    y32 = ops.conv2d_fwd(x, w, None, *geo).get()
+    _hip.set_conv_math('bf16')
+    try:
+        want = (ops.conv2d_fwd(x, w, None, *geo).get(), ops.conv2d_dgrad(gy, w, None, (h, h), *geo).get(),
+                ops.conv2d_wgrad(x, gy, (k, c, 3, 3), *geo).get())
+    finally:
+        _hip.set_conv_math('f32')
+    for got, ref in zip((y, dx, dw), want):
+        np.testing.assert_array_equal(got.get(), ref)
+    assert np.abs(y.get() - y32).max() > 0                       # really bf16
+    np.testing.assert_array_equal(ops.conv2d_fwd(x, w, None, *geo).get(), y32)   # and float32 for everybody else
+
+
 def test_module_api_switch():
     import pytortto_amd as tt
     tt.manual_seed(0)
