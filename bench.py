@@ -106,6 +106,12 @@ def traffic_per_launch(prefixes, launches_per_step=None):
 BN_SHAPES = [(64, 256, 56, 56), (128, 64, 112, 112)]
 
 
+def progress(text):
+    """A line on stderr (stdout carries the one JSON line): long phases, the host-side baseline above
+    all, say that they are alive."""
+    print(f'[bench] {text}', file=sys.stderr, flush=True)
+
+
 def conv_flops(n, c, h, k, r, s, p):
     q = (h + 2 * p - r) // s + 1
     return 2.0 * n * k * c * r * r * q * q, q
@@ -541,6 +547,7 @@ def cpu_baseline_conv(batch):
         oracle.convolution_backward(dy, x, xpad, w, (s, s), (p, p), (1, 1), 1, need=(True, True, False))
         seconds += time.perf_counter() - t0
         flops += 3 * f
+        progress(f'cpu baseline, batch {batch}: {c}x{h}x{h}->{k} k{r} s{s} done, {seconds:.1f} s so far')
     return flops, seconds
 
 
@@ -652,6 +659,7 @@ def main():
             for _ in range(l.count):
                 l.run(call)
 
+    progress('calibration probes, then the convolution step')
     # ---- what the device sustains on the two bounding resources, measured in this run ----------
     # (first: 0.2 s of dense matrix work and 8 GiB of streaming also bring the device from idle to
     # its sustained clocks before anything is timed; with 3 warm-up steps alone the first timed
@@ -671,9 +679,11 @@ def main():
     n_wg, ms_wg = prof['conv_wgrad']
     wgrad_tflops = flops_per_pass * args.steps / (ms_wg * 1e-3) / 1e12
     kernel_ms = {k: round(v[1] / args.steps, 4) for k, v in prof.items() if v[0]}
+    progress('per-layer table of the 23 shapes')
     layer_rows = None if args.no_per_layer else per_layer_table(_hip, call, layers, 20)
     c1_gpu = None if args.no_per_layer else single_layer_config(_hip, call, rng)   # (kept out of profiling runs)
 
+    progress('convolution step with bf16 arithmetic')
     # optional reduced-precision variant, reported separately and never part of `value`: the three
     # passes on bf16 MFMA (operands rounded inside the kernels, fp32 accumulation and tensors)
     _hip.set_conv_math('bf16')
@@ -704,6 +714,7 @@ def main():
     del layers
     call('tt_empty_cache')
 
+    progress('BatchNorm shapes')
     # ---- BatchNorm2d training fwd+bwd -----------------------------------------------------------
     bns = [BnLayer(s, rng) for s in BN_SHAPES]
     bn_bytes = sum(8 * b.bytes for b in bns)
@@ -728,6 +739,7 @@ def main():
     del bns
     call('tt_empty_cache')
 
+    progress('MaxPool2d and elementwise kernels')
     # ---- rows either side of the path: MaxPool2d (ResNet-50 stem pooling) and the activations ---
     pool_shape, pool_args = (BATCH, 64, 112, 112), (3, 3, 2, 2, 1, 1, 1, 1)
     px = hiparray(rng.standard_normal(pool_shape, dtype=np.float32))
@@ -764,6 +776,7 @@ def main():
     del px, py, ptap, pdx
     call('tt_empty_cache')
 
+    progress('whole ResNet-50 training step')
     # ---- the whole network through the module API ---------------------------------------------
     model = None
     if not args.no_model_step:
@@ -783,6 +796,7 @@ def main():
                                         'loss_first_last': [round(b_losses[0], 4), round(b_losses[-1], 4)]}
         call('tt_empty_cache')
 
+    progress('PreAct-ResNet-18 and DCGAN stacks')
     # ---- the other two stack configurations: per layer, then whole stacks through the module API ---
     stack_rows = {}
     if not args.no_per_layer:
@@ -825,6 +839,7 @@ def main():
     elif stack_rows:
         stacks = {k: {'per_layer': v} for k, v in stack_rows.items()}
 
+    progress('CPU baseline (oracle on the host cores)')
     # ---- CPU baseline (oracle on the host cores) -------------------------------------------------
     cpu_conv = cpu_bn = None
     if not args.no_cpu_baseline:
