@@ -104,15 +104,28 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
  * both operands are rounded to bfloat16 (nearest even) on their way into
  * v_mfma_f32_32x32x16_bf16 and products are accumulated in float32 (the weight gradient's
  * partial sums are still combined in float64); results differ from the float32 ones by about
- * 2^-8 of the operands' magnitude per term.  It applies to tt_conv2d_fwd_f32,
+ * 2^-8 of the operands' magnitude per term.
+ * TT_CONV_MATH_BF16X3 is float32 arithmetic on the bf16 matrix pipe, which is sixteen times as wide
+ * as the float32 one: inside the kernel every operand element becomes three bfloat16 terms that add
+ * up to it exactly (each the bf16 nearest to what the terms before it leave), and six
+ * v_mfma_f32_32x32x16_bf16 per product step accumulate in float32 every product of terms except the
+ * three smallest, which together stay below 2^-24 of the product (2^-27 in the root mean square):
+ * no more than rounding the product to float32 once.  Results meet the same tolerances as TT_CONV_MATH_F32 (they differ from it as two
+ * float32 summation orders do); non-finite operands and magnitudes above 3.38e38 (which round to a
+ * bf16 infinity) give NaN where float32 would give an infinity.  Launches it does not pay for
+ * (fewer tiles than compute units, strided input gradients, short weight-gradient reductions,
+ * kernels beyond 31 taps) run on the float32 instructions.
+ * The modes apply to tt_conv2d_fwd_f32,
  * tt_conv2d_dgrad_f32 and tt_conv2d_wgrad_f32.  The setting is process-wide and applies to
- * later calls of every caller; the *_bf16 entry points below select it per call instead. */
-enum { TT_CONV_MATH_F32 = 0, TT_CONV_MATH_BF16 = 1 };
+ * later calls of every caller; the *_bf16 and *_bf16x3 entry points below select a mode per call
+ * instead. */
+enum { TT_CONV_MATH_F32 = 0, TT_CONV_MATH_BF16 = 1, TT_CONV_MATH_BF16X3 = 2 };
 int tt_set_conv_math(int mode);
 int tt_get_conv_math(int* mode);   /* host pointer */
-/* The same three passes with bf16 matrix arithmetic for one call, whatever the process-wide mode is
- * (arguments as tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 / tt_conv2d_wgrad_f32 below; tensors are
- * float32): for callers that must not change what other callers of the library compute. */
+/* The same three passes with bf16 (*_bf16) or three-term (*_bf16x3) matrix arithmetic for one call,
+ * whatever the process-wide mode is (arguments as tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 /
+ * tt_conv2d_wgrad_f32 below; tensors are float32): for callers that must not change what other
+ * callers of the library compute. */
 int tt_conv2d_fwd_bf16(const float* x, const float* w, const float* bias, float* y,
                        int N, int C, int H, int W, int K, int R, int S,
                        int sh, int sw, int ph, int pw, int dh, int dw, int groups);
@@ -122,6 +135,15 @@ int tt_conv2d_dgrad_bf16(const float* dy, const float* w, const float* bias, flo
 int tt_conv2d_wgrad_bf16(const float* x, const float* dy, float* dw,
                          int N, int C, int H, int W, int K, int R, int S,
                          int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q);
+int tt_conv2d_fwd_bf16x3(const float* x, const float* w, const float* bias, float* y,
+                         int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int ph, int pw, int dh, int dw, int groups);
+int tt_conv2d_dgrad_bf16x3(const float* dy, const float* w, const float* bias, float* dx,
+                           int N, int C, int Hx, int Wx, int K, int R, int S,
+                           int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q);
+int tt_conv2d_wgrad_bf16x3(const float* x, const float* dy, float* dw,
+                           int N, int C, int H, int W, int K, int R, int S,
+                           int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q);
 
 /* Tuning threshold of tt_conv2d_dgrad_f32 for strided layers with very few input channels (the
  * ResNet stem, the output layer of a transposed generator), no counterpart in the reference.
@@ -211,7 +233,8 @@ int tt_conv2d_selftest_raise_async_error(void);
 int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* per);
 /* The plan of the last single matrix-product launch made by tt_conv2d_fwd_f32 / _dgrad_f32 (host
  * pointer to 8 ints): tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent
- * grid (0 = one tile per block, -1 = one tile per block on the bf16-first kernels), tiles computed
+ * grid (0 = one tile per block; -1, -3 = one tile per block on the bf16-first kernels with one or
+ * three bf16 terms per operand element), tiles computed
  * whole, blocks sharing the remaining tiles'
  * reductions, addressing mode.  Tests use it to compare the images where the shared tiles begin. */
 int tt_conv2d_last_launch(int* plan8);
@@ -227,7 +250,9 @@ int tt_conv2d_last_launch(int* plan8);
  * most 1024 (1, the default) or whenever those kernels support the geometry (2: small test shapes);
  * 0 keeps every launch on the float32 kernels' bf16 instantiations, which also serve the launches
  * the former do not take.  Both compute the same thing: the convolution of
- * the bf16-rounded operands in float32. */
+ * the bf16-rounded operands in float32.  With TT_CONV_MATH_BF16X3 the same switch decides between
+ * the three-term kernels and the float32 instructions: 1 = where a launch has a tile per compute
+ * unit (weight gradient: at least 8192 pixels to sum over), 2 = wherever supported, 0 = never. */
 int tt_conv2d_bf16_first_enable(int on);
 int tt_conv2d_last_wgrad_launch(int* plan4);
 int tt_conv2d_wgrad_force_occupancy(int blocks);

@@ -38,10 +38,12 @@ class cuda:
 
     @staticmethod
     def set_conv_math(mode):
-        """Not in the reference (float32 throughout): ``'f32'`` (default) or ``'bf16'`` -- the three
+        """Not in the reference (float32 throughout): ``'f32'`` (default), ``'bf16'`` -- the three
         convolution passes with operands rounded to bfloat16 inside the kernels and float32
-        accumulation.  Tensors stay float32; results then differ from the float32 path by a few 1e-3
-        of their magnitude."""
+        accumulation; tensors stay float32, results then differ from the float32 path by a few 1e-3
+        of their magnitude -- or ``'bf16x3'``: float32 arithmetic carried out on the bf16 matrix
+        instructions (three exact bf16 terms per operand element), which meets the float32 path's
+        tolerances and is faster on layers with at least one tile per compute unit."""
         _hip.set_conv_math(mode)
 
     @staticmethod

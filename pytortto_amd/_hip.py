@@ -44,6 +44,9 @@ PROTOTYPES = {
     'tt_conv2d_fwd_bf16': [_P, _P, _P, _P] + [_I] * 14,
     'tt_conv2d_dgrad_bf16': [_P, _P, _P, _P] + [_I] * 16,
     'tt_conv2d_wgrad_bf16': [_P, _P, _P] + [_I] * 16,
+    'tt_conv2d_fwd_bf16x3': [_P, _P, _P, _P] + [_I] * 14,
+    'tt_conv2d_dgrad_bf16x3': [_P, _P, _P, _P] + [_I] * 16,
+    'tt_conv2d_wgrad_bf16x3': [_P, _P, _P] + [_I] * 16,
     'tt_conv2d_check_tables_fwd_f32': [_I] * 14,
     'tt_conv2d_check_tables_dgrad_f32': [_I] * 16,
     'tt_conv2d_check_tables_wgrad_f32': [_I] * 16,
@@ -254,13 +257,15 @@ def probe_hbm(nbytes=2 << 30):
     return rd.value, cp.value
 
 
-CONV_MATH = {'f32': 0, 'bf16': 1}
+CONV_MATH = {'f32': 0, 'bf16': 1, 'bf16x3': 2}
 
 
 def set_conv_math(mode):
-    """Matrix arithmetic of the three convolution passes: 'f32' (default, the mode that meets
-    the reference's tolerances) or 'bf16' (operands rounded to bfloat16 inside the kernel, float32
-    accumulation; tensors stay float32)."""
+    """Matrix arithmetic of the three convolution passes: 'f32' (default: float32 matrix
+    instructions), 'bf16' (operands rounded to bfloat16 inside the kernel, float32 accumulation;
+    tensors stay float32) or 'bf16x3' (float32 arithmetic on the bf16 matrix pipe: every operand
+    element as three bf16 terms that add up to it exactly, six products per step; meets the same
+    tolerances as 'f32')."""
     if mode not in CONV_MATH:
         raise ValueError(f"conv math must be one of {sorted(CONV_MATH)}, got {mode!r}")
     call('tt_set_conv_math', CONV_MATH[mode])

@@ -853,6 +853,9 @@ bool wants_stream_k(long long tiles, int chunks, int groups) {
 // The bf16 kernels are bound by their fetch path, not by the matrix pipe: smaller tiles fetch more
 // per FLOP and lose there.
 bool bf16_math() { return tt::conv_math() == TT_CONV_MATH_BF16; }
+// float32 arithmetic on the bf16 matrix pipe (three bf16 terms per operand element): launches the
+// bf16-first kernels take run there, every other launch on the float32 kernels.
+bool split_math() { return tt::conv_math() == TT_CONV_MATH_BF16X3; }
 
 // Blocks of a persistent launch: the bf16 kernels hide their loads with a third block per CU
 // (measured: 3 % faster than two, four do not fit the register file).
@@ -1037,6 +1040,12 @@ int g_last_launch[8] = {};
 bool g_bf16_first = true;
 bool g_bf16_first_always = false;   // tests: also where the tile-count rule would keep the other kernels
 
+}  // namespace
+namespace tt {
+bool conv_bf16_kernels_forced() { return g_bf16_first_always; }
+}
+namespace {
+
 int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_partial) {
   tt::ProfScope prof(prof_id);
   p.tilesI = p.Ipad / t.bm;
@@ -1065,12 +1074,23 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
   // long reduction stay on the stream-K instantiations (measured per layer: 1.2-1.8 times faster
   // where taken, up to 2 times slower on 100 tiles of 144 chunks).
   const int bf_tiles = (p.Ipad / t.bm) * ceil_div(p.M, 128);
+  int bf_bm = 0, bf_terms = 1;   // tile rows and bf16 terms per element of the launch they take (0: not taken)
   if (bf16_math() && g_bf16_first && bf16_first_supported(p, groups, t.bm) &&
       ((long long)bf_tiles * groups >= cus() || p.Kred <= 1024 || g_bf16_first_always)) {
-    const int tiles = bf_tiles;
-    const int plan[8] = {t.bm, 128, tiles, p.Ipad / t.bm, -1, tiles, 0, p.mode};   // -1: the bf16-first kernels
+    bf_bm = t.bm;
+  } else if (split_math() && g_bf16_first && bf16_first_supported(p, groups, t.bm) &&
+             ((long long)bf_tiles * groups >= cus() || g_bf16_first_always)) {
+    // float32 arithmetic on the bf16 pipe is bound by the matrix pipe again and shares no reduction
+    // between blocks: taken where every compute unit gets a tile; other launches stay on the float32
+    // instructions (64-row tiles for them were measured no faster than those).
+    bf_bm = t.bm;
+    bf_terms = 3;
+  }
+  if (bf_bm > 0) {
+    const int tiles = (p.Ipad / bf_bm) * ceil_div(p.M, 128);
+    const int plan[8] = {bf_bm, 128, tiles, p.Ipad / bf_bm, -bf_terms, tiles, 0, p.mode};   // -1, -3: the bf16-first kernels, by terms
     std::copy(plan, plan + 8, g_last_launch);
-    bf16_first_launch(p, groups, t.bm, st);
+    bf16_first_launch(p, groups, bf_bm, bf_terms, st);
     TT_LAUNCH_CHECK();
     return 0;
   }
@@ -1444,7 +1464,7 @@ static int conv2d_fwd(const float* x, const float* w, const float* bias, float* 
   const int M = N * P * Q;
   const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
   const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
-  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ, true, plain && KQ / kBKQ <= 32 && !bf16_math());
+  const TileChoice t = choose_tile(Kg, M, groups, KQ / kBKQ, true, plain && KQ / kBKQ <= 32 && !bf16_math() && !split_math());
   const int Ipad = ceil_div(Kg, t.bm) * t.bm;
 
   const size_t wp_bytes = align_up(sizeof(floatx4) * (size_t)groups * KQ * Ipad, 256);
@@ -1699,7 +1719,7 @@ static int conv2d_dgrad(const float* dy, const float* w, const float* bias, floa
       const int KQ = ceil_div(Kred, 4 * kBKQ) * kBKQ;
       const bool plain = R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0;
       const TileChoice t = choose_tile(Cg, M, groups, KQ / kBKQ, allow_stream_k,
-                                       (plain && KQ / kBKQ <= 32 && !bf16_math()) || !allow_stream_k);
+                                       (plain && KQ / kBKQ <= 32 && !bf16_math() && !split_math()) || !allow_stream_k);
       const int Ipad = ceil_div(Cg, t.bm) * t.bm;
       floatx4* wp = (floatx4*)((char*)ws + wp_bytes * slot);
       Igemm p{};

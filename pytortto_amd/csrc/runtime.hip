@@ -288,7 +288,7 @@ int tt_memset(void* dst_dev, int byte_value, size_t bytes) {
 
 int tt_set_conv_math(int mode) {
   TT_API_LOCK();
-  TT_REQUIRE(mode == TT_CONV_MATH_F32 || mode == TT_CONV_MATH_BF16, "tt_set_conv_math: unknown mode %d", mode);
+  TT_REQUIRE(mode == TT_CONV_MATH_F32 || mode == TT_CONV_MATH_BF16 || mode == TT_CONV_MATH_BF16X3, "tt_set_conv_math: unknown mode %d", mode);
   S().conv_math = mode;
   return 0;
 }
@@ -300,14 +300,17 @@ int tt_get_conv_math(int* mode) {
   return 0;
 }
 
-// The three convolution passes with bf16 matrix arithmetic for this call only, whatever the
+// The three convolution passes with another matrix arithmetic for this call only, whatever the
 // process-wide mode is: the mode is switched under the API lock, which this thread holds for the
 // whole call, so no other caller can see the switch.
 namespace {
-struct ScopedBf16 {
+struct ScopedMath {
   int saved;
-  ScopedBf16() : saved(S().conv_math) { S().conv_math = TT_CONV_MATH_BF16; }
-  ~ScopedBf16() { S().conv_math = saved; }
+  explicit ScopedMath(int mode) : saved(S().conv_math) { S().conv_math = mode; }
+  ~ScopedMath() { S().conv_math = saved; }
+};
+struct ScopedBf16 : ScopedMath {
+  ScopedBf16() : ScopedMath(TT_CONV_MATH_BF16) {}
 };
 }  // namespace
 
@@ -329,6 +332,27 @@ int tt_conv2d_wgrad_bf16(const float* x, const float* dy, float* dw, int N, int 
                          int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
   TT_API_LOCK();
   ScopedBf16 mode;
+  return tt_conv2d_wgrad_f32(x, dy, dw, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw_, groups, P, Q);
+}
+
+int tt_conv2d_fwd_bf16x3(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K,
+                         int R, int S_, int sh, int sw, int ph, int pw, int dh, int dw, int groups) {
+  TT_API_LOCK();
+  ScopedMath mode(TT_CONV_MATH_BF16X3);
+  return tt_conv2d_fwd_f32(x, w, bias, y, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw, groups);
+}
+
+int tt_conv2d_dgrad_bf16x3(const float* dy, const float* w, const float* bias, float* dx, int N, int C, int Hx, int Wx,
+                           int K, int R, int S_, int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q) {
+  TT_API_LOCK();
+  ScopedMath mode(TT_CONV_MATH_BF16X3);
+  return tt_conv2d_dgrad_f32(dy, w, bias, dx, N, C, Hx, Wx, K, R, S_, sh, sw, ph, pw, dh, dw, groups, P, Q);
+}
+
+int tt_conv2d_wgrad_bf16x3(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S_,
+                           int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
+  TT_API_LOCK();
+  ScopedMath mode(TT_CONV_MATH_BF16X3);
   return tt_conv2d_wgrad_f32(x, dy, dw, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw_, groups, P, Q);
 }
 
