@@ -112,9 +112,10 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
  * three smallest, which together stay below 2^-24 of the product (2^-27 in the root mean square):
  * no more than rounding the product to float32 once.  Results meet the same tolerances as TT_CONV_MATH_F32 (they differ from it as two
  * float32 summation orders do); non-finite operands and magnitudes above 3.38e38 (which round to a
- * bf16 infinity) give NaN where float32 would give an infinity.  Launches it does not pay for
- * (fewer tiles than compute units, strided input gradients, short weight-gradient reductions,
- * kernels beyond 31 taps) run on the float32 instructions.
+ * bf16 infinity) give NaN where float32 would give an infinity.  Forward and input gradient run
+ * that way for every geometry; weight gradients it does not pay for (fewer than 8192 pixels to sum
+ * over, 64-row tiles of kernels larger than 1x1, kernels of 32 to 63 taps) run on the float32
+ * instructions.
  * The modes apply to tt_conv2d_fwd_f32,
  * tt_conv2d_dgrad_f32 and tt_conv2d_wgrad_f32.  The setting is process-wide and applies to
  * later calls of every caller; the *_bf16 and *_bf16x3 entry points below select a mode per call
@@ -219,7 +220,9 @@ int tt_conv2d_check_tables_selftest_wgrad(void);
  * other; that is safe only while the whole grid is resident, so the library asks the device how
  * many blocks of each such kernel a compute unit holds and launches one tile per block instead
  * where it is too few.
- *   tt_conv2d_stream_k_blocks_per_cu: the smallest answer over all such kernels (host pointer).
+ *   tt_conv2d_stream_k_blocks_per_cu: the smallest answer over all such kernels of one matrix
+ *     arithmetic (bf16 = 0: float32 instructions, 1: TT_CONV_MATH_BF16, 3: TT_CONV_MATH_BF16X3, which
+ *     like the float32 ones runs two blocks per compute unit; host pointer).
  *   tt_conv2d_stream_k_force_occupancy: pretend the answer is `blocks` (-1: ask the device).
  *   tt_conv2d_selftest_raise_async_error: a one-thread kernel sets the word that a block sets when
  *     its bounded wait for another block runs out; the next tt_sync() / tt_memcpy_d2h() returns
@@ -233,10 +236,11 @@ int tt_conv2d_selftest_raise_async_error(void);
 int tt_conv2d_images_per_run(int N, long long image_a, long long image_b, int* per);
 /* The plan of the last single matrix-product launch made by tt_conv2d_fwd_f32 / _dgrad_f32 (host
  * pointer to 8 ints): tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent
- * grid (0 = one tile per block; -1, -3 = one tile per block on the bf16-first kernels with one or
- * three bf16 terms per operand element), tiles computed
+ * grid (0 = one tile per block, -1 = one tile per block on the bf16-first kernels), tiles computed
  * whole, blocks sharing the remaining tiles'
- * reductions, addressing mode.  Tests use it to compare the images where the shared tiles begin. */
+ * reductions, addressing mode | terms << 8 with terms = bf16 terms per operand element of the matrix
+ * instructions used (0 = float32 instructions, 1 = TT_CONV_MATH_BF16, 3 = TT_CONV_MATH_BF16X3).
+ * Tests use it to compare the images where the shared tiles begin. */
 int tt_conv2d_last_launch(int* plan8);
 /* The same for the weight gradient, whose blocks add each other's partial sums inside the kernel
  * when the device holds the whole grid at once and leave them to a second kernel otherwise:
@@ -250,9 +254,8 @@ int tt_conv2d_last_launch(int* plan8);
  * most 1024 (1, the default) or whenever those kernels support the geometry (2: small test shapes);
  * 0 keeps every launch on the float32 kernels' bf16 instantiations, which also serve the launches
  * the former do not take.  Both compute the same thing: the convolution of
- * the bf16-rounded operands in float32.  With TT_CONV_MATH_BF16X3 the same switch decides between
- * the three-term kernels and the float32 instructions: 1 = where a launch has a tile per compute
- * unit (weight gradient: at least 8192 pixels to sum over), 2 = wherever supported, 0 = never. */
+ * the bf16-rounded operands in float32.  With TT_CONV_MATH_BF16X3, 2 sends every weight gradient
+ * the three-term kernels support to them, whatever the size rule says. */
 int tt_conv2d_bf16_first_enable(int on);
 int tt_conv2d_last_wgrad_launch(int* plan4);
 int tt_conv2d_wgrad_force_occupancy(int blocks);

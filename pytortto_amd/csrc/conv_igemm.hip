@@ -193,9 +193,36 @@ __device__ __forceinline__ floatx4 load_coherent(__amdgpu_buffer_rsrc_t rsrc, in
   return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, kSystemScope));
 }
 
+// Eight float32 values (a lane's k values of one 16-deep matrix step) as three vectors of bfloat16
+// terms that add up to them exactly: term i of value v is the bf16 nearest to v minus the terms
+// before it.
+__device__ __forceinline__ void three_terms(const floatx4 lo, const floatx4 hi, bf16x8 (&out)[3]) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+  const float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  unsigned t[3][4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    float e = v[2 * q], o = v[2 * q + 1];   // the pair shares a register of every term
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const bf16x2 pair = {(__bf16)e, (__bf16)o};
+      t[i][q] = __builtin_bit_cast(unsigned, pair);
+      if (i < 2) {
+        e -= as_float(t[i][q] << 16);
+        o -= as_float(t[i][q] & 0xffff0000u);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 3; ++i) out[i] = __builtin_bit_cast(bf16x8, uintx4{t[i][0], t[i][1], t[i][2], t[i][3]});
+}
+
 // The kernel body: `block_x` is the block's index among the blocks of launch `p` (a launch may
 // be one of several that share a grid, see igemm_multi_f32).
-template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT, bool BF>
+// BF: 0 = float32 matrix instructions; 1 = operands rounded to bfloat16; 3 = float32 arithmetic on the
+// bf16 matrix instructions (three bf16 terms per operand element, six products per step).
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT, int BF>
 __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   static_assert(WM * WN == 4, "four waves per block");
   constexpr bool GEMM = MODE == kModeGemm, BUF = MODE != kModeCompare;
@@ -426,7 +453,37 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
   // sched_barrier pins this order; the compiler otherwise sinks the loads below the MFMAs.
   constexpr int T = 8 * MT * NT;
   auto chunk_body = [&](const int set, const int nchunk, const int nnchunk) __attribute__((always_inline)) {
-    if constexpr (BF) {
+    if constexpr (BF == 3) {
+      // float32 arithmetic on the bf16 matrix instructions.  Every operand value v read from LDS
+      // becomes three bfloat16 terms, t0 = bf16(v), t1 = bf16(v - t0), t2 = bf16(v - t0 - t1) (nearest
+      // even; both differences are exact in float32), so that v = t0 + t1 + t2 exactly, and six
+      // v_mfma_f32_32x32x16_bf16 per accumulator add up every product of terms except (t1,t2), (t2,t1)
+      // and (t2,t2), which together stay below 2^-24 of the product: half an ulp of it, what rounding
+      // it to float32 once would cost.  bf16 x bf16 is exact in float32; accumulation is float32.
+      // Six instructions of 32 cycles replace eight of 64; the price is the conversion, about 5.5
+      // vector instructions per value, which issue next to the matrix instructions of the other
+      // wave on the SIMD.
+      load_all(nchunk);
+      __builtin_amdgcn_sched_barrier(0);
+      bf16x8 a[MT][3], b[NT][3];
+#pragma unroll
+      for (int x = 0; x < MT; ++x) three_terms(opA[set][0][x], opA[set][1][x], a[x]);
+#pragma unroll
+      for (int y = 0; y < NT; ++y) three_terms(opB[set][0][y], opB[set][1][y], b[y]);
+      constexpr int ta[6] = {2, 0, 1, 1, 0, 0}, tb[6] = {0, 2, 1, 0, 1, 0};   // smallest products first
+#pragma unroll
+      for (int o = 0; o < 6; ++o)
+#pragma unroll
+        for (int x = 0; x < MT; ++x)
+#pragma unroll
+          for (int y = 0; y < NT; ++y)
+            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x][ta[o]], b[y][tb[o]], acc[x][y], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      store_all(set ^ 1);
+      __syncthreads();
+      read_ops(set ^ 1, set ^ 1);
+      load_tab(nnchunk);
+    } else if constexpr (BF == 1) {
       // bf16 matrix instructions: one v_mfma_f32_32x32x16_bf16 per accumulator contracts the whole
       // chunk (a lane's two quads are its eight k values, the same ones for both operands), so a
       // chunk's matrix time is a sixteenth of the fp32 one and there is no shadow to weave the
@@ -795,12 +852,17 @@ __device__ __forceinline__ void igemm_body(const Igemm& p, const int block_x) {
 
 template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
 __global__ __launch_bounds__(kThreads, 2) void igemm_f32(const Igemm p) {
-  igemm_body<WM, WN, MT, NT, SK, MODE, AT, false>(p, (int)blockIdx.x);
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT, 0>(p, (int)blockIdx.x);
 }
 // The same launch on bf16 matrix instructions (tt_set_conv_math); three blocks per CU.
 template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
 __global__ __launch_bounds__(kThreads, 3) void igemm_bf16(const Igemm p) {
-  igemm_body<WM, WN, MT, NT, SK, MODE, AT, true>(p, (int)blockIdx.x);
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT, 1>(p, (int)blockIdx.x);
+}
+// The same launch in float32 arithmetic carried out on the bf16 matrix instructions; two blocks per CU.
+template <int WM, int WN, int MT, int NT, bool SK, int MODE, bool AT>
+__global__ __launch_bounds__(kThreads, 2) void igemm_bf16x3(const Igemm p) {
+  igemm_body<WM, WN, MT, NT, SK, MODE, AT, 3>(p, (int)blockIdx.x);
 }
 
 // Several data-parallel launches in one grid (the stride-parity classes of a strided input
@@ -815,13 +877,19 @@ template <int WM, int WN, int MT, int NT, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void igemm_multi_f32(const IgemmMulti m) {
   int ci = 0;
   while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
-  igemm_body<WM, WN, MT, NT, false, MODE, false, false>(m.c[ci], (int)blockIdx.x - m.first[ci]);
+  igemm_body<WM, WN, MT, NT, false, MODE, false, 0>(m.c[ci], (int)blockIdx.x - m.first[ci]);
 }
 template <int WM, int WN, int MT, int NT, int MODE>
 __global__ __launch_bounds__(kThreads, 3) void igemm_multi_bf16(const IgemmMulti m) {
   int ci = 0;
   while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
-  igemm_body<WM, WN, MT, NT, false, MODE, false, true>(m.c[ci], (int)blockIdx.x - m.first[ci]);
+  igemm_body<WM, WN, MT, NT, false, MODE, false, 1>(m.c[ci], (int)blockIdx.x - m.first[ci]);
+}
+template <int WM, int WN, int MT, int NT, int MODE>
+__global__ __launch_bounds__(kThreads, 2) void igemm_multi_bf16x3(const IgemmMulti m) {
+  int ci = 0;
+  while (ci + 1 < m.n && (int)blockIdx.x >= m.first[ci + 1]) ++ci;
+  igemm_body<WM, WN, MT, NT, false, MODE, false, 3>(m.c[ci], (int)blockIdx.x - m.first[ci]);
 }
 
 // ---- host side -------------------------------------------------------------------------------------
@@ -856,6 +924,8 @@ bool bf16_math() { return tt::conv_math() == TT_CONV_MATH_BF16; }
 // float32 arithmetic on the bf16 matrix pipe (three bf16 terms per operand element): launches the
 // bf16-first kernels take run there, every other launch on the float32 kernels.
 bool split_math() { return tt::conv_math() == TT_CONV_MATH_BF16X3; }
+// bf16 terms per operand element of the matrix instructions in use (0: float32 instructions)
+int math_terms() { return bf16_math() ? 1 : split_math() ? 3 : 0; }
 
 // Blocks of a persistent launch: the bf16 kernels hide their loads with a third block per CU
 // (measured: 3 % faster than two, four do not fit the register file).
@@ -893,13 +963,14 @@ size_t sk_workspace_bytes() { return (size_t)sk_launch_blocks() * 128 * 128 * si
 // instantiation is asked once (registers and LDS of the compiled kernel decide it); an
 // instantiation that cannot hold that many is launched data-parallel instead, one tile per block:
 // a register-count regression then costs speed, never a stalled launch.
-template <int WM, int WN, int MT, int NT, int MODE, bool AT, bool BFK>
+template <int WM, int WN, int MT, int NT, int MODE, bool AT, int BFK>
 int sk_resident_blocks_per_cu() {
   static int cached = -1;
   if (cached < 0) {
     int n = 0;
     hipError_t e;
-    if constexpr (BFK) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_bf16<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
+    if constexpr (BFK == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_bf16<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
+    else if constexpr (BFK == 3) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_bf16x3<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
     else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, igemm_f32<WM, WN, MT, NT, true, MODE, AT>, kThreads, 0);
     if (e != hipSuccess) {
       (void)hipGetLastError();
@@ -914,25 +985,30 @@ int g_sk_forced_occupancy = -1;   // >= 0: pretend every instantiation holds thi
 // Returns whether the persistent (stream-K) grid was launched.
 template <int WM, int WN, int MT, int NT, int MODE, bool AT>
 bool launch_mode(const Igemm& p, int groups, int sk_blocks, hipStream_t st) {
-  const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
+  const int math = tt::conv_math();
+  const bool bf = math == TT_CONV_MATH_BF16, x3 = math == TT_CONV_MATH_BF16X3;
   if (sk_blocks > 0) {
-    int held = bf ? sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, true>()
-                  : sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, false>();
+    int held = bf   ? sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, 1>()
+               : x3 ? sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, 3>()
+                    : sk_resident_blocks_per_cu<WM, WN, MT, NT, MODE, AT, 0>();
     if (g_sk_forced_occupancy >= 0) held = g_sk_forced_occupancy;
     if ((long long)held * cus() < sk_blocks) sk_blocks = 0;   // the data-parallel launch ignores the stream-K fields
   }
   if (sk_blocks > 0) {
     if (bf) igemm_bf16<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
+    else if (x3) igemm_bf16x3<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
     else igemm_f32<WM, WN, MT, NT, true, MODE, AT><<<dim3(sk_blocks, 1), kThreads, 0, st>>>(p);
   } else if (bf) {
     igemm_bf16<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
+  } else if (x3) {
+    igemm_bf16x3<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   } else {
     igemm_f32<WM, WN, MT, NT, false, MODE, AT><<<dim3(p.tiles, groups), kThreads, 0, st>>>(p);
   }
   return sk_blocks > 0;
 }
 // smallest number of resident blocks per CU over every stream-K instantiation of one tile shape
-template <int WM, int WN, int MT, int NT, bool BFK>
+template <int WM, int WN, int MT, int NT, int BFK>
 int sk_min_resident() {
   const int all[] = {sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeGemm, true, BFK>(),
                      sk_resident_blocks_per_cu<WM, WN, MT, NT, kModeGemm, false, BFK>(),
@@ -944,7 +1020,7 @@ int sk_min_resident() {
   for (int v : all) lo = v < lo ? v : lo;
   return lo;
 }
-template <bool BFK>
+template <int BFK>
 int sk_min_resident_all() {
   const int all[] = {sk_min_resident<2, 2, 2, 2, BFK>(), sk_min_resident<1, 4, 2, 2, BFK>(),
                      sk_min_resident<1, 4, 1, 2, BFK>(), sk_min_resident<2, 2, 1, 1, BFK>()};
@@ -1074,28 +1150,21 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
   // long reduction stay on the stream-K instantiations (measured per layer: 1.2-1.8 times faster
   // where taken, up to 2 times slower on 100 tiles of 144 chunks).
   const int bf_tiles = (p.Ipad / t.bm) * ceil_div(p.M, 128);
-  int bf_bm = 0, bf_terms = 1;   // tile rows and bf16 terms per element of the launch they take (0: not taken)
+  int bf_bm = 0;   // tile rows of the launch they take (0: not taken)
   if (bf16_math() && g_bf16_first && bf16_first_supported(p, groups, t.bm) &&
       ((long long)bf_tiles * groups >= cus() || p.Kred <= 1024 || g_bf16_first_always)) {
     bf_bm = t.bm;
-  } else if (split_math() && g_bf16_first && bf16_first_supported(p, groups, t.bm) &&
-             ((long long)bf_tiles * groups >= cus() || g_bf16_first_always)) {
-    // float32 arithmetic on the bf16 pipe is bound by the matrix pipe again and shares no reduction
-    // between blocks: taken where every compute unit gets a tile; other launches stay on the float32
-    // instructions (64-row tiles for them were measured no faster than those).
-    bf_bm = t.bm;
-    bf_terms = 3;
   }
   if (bf_bm > 0) {
     const int tiles = (p.Ipad / bf_bm) * ceil_div(p.M, 128);
-    const int plan[8] = {bf_bm, 128, tiles, p.Ipad / bf_bm, -bf_terms, tiles, 0, p.mode};   // -1, -3: the bf16-first kernels, by terms
+    const int plan[8] = {bf_bm, 128, tiles, p.Ipad / bf_bm, -1, tiles, 0, p.mode | 1 << 8};   // -1: the bf16-first kernels
     std::copy(plan, plan + 8, g_last_launch);
-    bf16_first_launch(p, groups, bf_bm, bf_terms, st);
+    bf16_first_launch(p, groups, bf_bm, st);
     TT_LAUNCH_CHECK();
     return 0;
   }
   const int plan[8] = {t.bm, t.bn, p.tiles, p.tilesI, t.sk_blocks, t.sk_blocks > 0 ? p.skDpTiles : p.tiles,
-                       t.sk_blocks > 0 ? p.skBlocks : 0, p.mode};
+                       t.sk_blocks > 0 ? p.skBlocks : 0, p.mode | math_terms() << 8};
   std::copy(plan, plan + 8, g_last_launch);
   bool persistent;
   if (t.bm == 128 && t.bn == 128)
@@ -1120,12 +1189,14 @@ int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_pa
 template <int WM, int WN, int MT, int NT>
 void launch_multi_config(const IgemmMulti& m, int groups, hipStream_t st) {
   const dim3 grid(m.first[m.n], groups);
-  const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
+  const bool bf = bf16_math(), x3 = split_math();
   if (m.c[0].mode == kModeTapMask) {
     if (bf) igemm_multi_bf16<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
+    else if (x3) igemm_multi_bf16x3<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
     else igemm_multi_f32<WM, WN, MT, NT, kModeTapMask><<<grid, kThreads, 0, st>>>(m);
   } else {
     if (bf) igemm_multi_bf16<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
+    else if (x3) igemm_multi_bf16x3<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
     else igemm_multi_f32<WM, WN, MT, NT, kModeCompare><<<grid, kThreads, 0, st>>>(m);
   }
 }
@@ -1138,7 +1209,7 @@ int launch_igemm_multi(IgemmMulti& m, int groups, TileChoice t, int prof_id) {
     p.tiles = p.tilesI * ceil_div(p.M, t.bn);
     m.first[i + 1] = m.first[i] + p.tiles;
   }
-  const int plan[8] = {t.bm, t.bn, m.first[m.n], 0, 0, m.first[m.n], 0, m.c[0].mode};   // several launches in one grid
+  const int plan[8] = {t.bm, t.bn, m.first[m.n], 0, 0, m.first[m.n], 0, m.c[0].mode | math_terms() << 8};   // several launches in one grid
   std::copy(plan, plan + 8, g_last_launch);
   hipStream_t st = tt::stream();
   if (t.bm == 128 && t.bn == 128)
@@ -1396,14 +1467,14 @@ int tt_set_conv_dense_cell_min_tiles(int tiles) {
 int tt_conv2d_stream_k_blocks_per_cu(int bf16, int* blocks) {
   TT_REQUIRE_INIT();
   TT_REQUIRE(blocks != nullptr, "tt_conv2d_stream_k_blocks_per_cu: null result pointer");
-  *blocks = bf16 ? sk_min_resident_all<true>() : sk_min_resident_all<false>();
+  *blocks = bf16 == 3 ? sk_min_resident_all<3>() : bf16 ? sk_min_resident_all<1>() : sk_min_resident_all<0>();
   return 0;
 }
 
 // Instrumentation (tests): the plan of the last single matrix-product launch of a forward or input
 // gradient call: {tile rows, tile columns (pixels), tiles, row tiles, blocks of the persistent grid
 // (0: one tile per block; -1: one tile per block on the bf16-first kernels), tiles computed whole (the rest share their reduction between blocks),
-// blocks sharing them, addressing mode}.  Pixel tile t starts at pixel (t / row tiles) * tile columns.
+// blocks sharing them, addressing mode | bf16 terms per operand element << 8 (0: float32 matrix instructions)}.  Pixel tile t starts at pixel (t / row tiles) * tile columns.
 int tt_conv2d_last_launch(int* plan8) {
   TT_API_LOCK();
   TT_REQUIRE(plan8 != nullptr, "tt_conv2d_last_launch: null result pointer");

@@ -37,20 +37,6 @@ __device__ __forceinline__ unsigned pack2(float lo, float hi) {
   return __builtin_bit_cast(unsigned, v);
 }
 
-// Two float32 values as PL pairs of bfloat16.  PL = 1: rounded to nearest even.  PL = 3: v = t0 + t1 + t2
-// exactly, every term the bf16 nearest to what the terms before it leave (each difference is exact in
-// float32: the remainder of a value rounded to 8 significant bits has at most 16).
-template <int PL>
-__device__ __forceinline__ void terms2(float lo, float hi, unsigned (&t)[PL]) {
-  t[0] = pack2(lo, hi);
-  if constexpr (PL == 3) {
-    const float l1 = lo - as_float(t[0] << 16), h1 = hi - as_float(t[0] & 0xffff0000u);
-    t[1] = pack2(l1, h1);
-    const float l2 = l1 - as_float(t[1] << 16), h2 = h1 - as_float(t[1] & 0xffff0000u);
-    t[2] = pack2(l2, h2);
-  }
-}
-
 // Column of a row / pixel inside an LDS line: one empty 16-byte unit after every sixteen, so that the
 // 8-byte writes of the transposing fetch (lanes four pixels apart) spread over the banks while reads
 // of 32 consecutive rows stay conflict-free.
@@ -64,21 +50,14 @@ constexpr int line_units(int n) { return n + n / 16 + 2; }
 //   kQuads: the repacked copy wp[k/4][row][4] of the float32 kernels
 constexpr int kRows = 0, kCols = 1, kQuads = 2;
 
-// PL = 1: operands rounded to bfloat16, LDS double-buffered, three blocks per compute unit.
-// PL = 3: float32 arithmetic on the bf16 matrix pipe: every operand element enters LDS as three bf16
-// terms that add up to it exactly, and the six products of terms that matter (the three left out are
-// below 2^-24 of the product, half an ulp of it) are accumulated in float32; one LDS buffer (two barriers per chunk), two
-// blocks per compute unit.
-template <int WM, int WN, int MT, int NT, bool GEMM, int AMODE, int PL>
-__global__ __launch_bounds__(kThreads, PL == 1 ? 3 : 2) void igemm_bf16_first(const Igemm p, const int tilesM) {
+template <int WM, int WN, int MT, int NT, bool GEMM, int AMODE>
+__global__ __launch_bounds__(kThreads, 3) void igemm_bf16_first(const Igemm p, const int tilesM) {
   static_assert(WM * WN == 4, "four waves per block");
-  static_assert(PL == 1 || PL == 3, "terms per operand element");
   constexpr int BM = WM * MT * 32, BN = WN * NT * 32;
   static_assert(BN == 128 && (BM == 128 || BM == 64), "tile shape");
   constexpr int ALINE = line_units(BM), BLINE = line_units(BN);
-  constexpr int NBUF = PL == 1 ? 2 : 1;
-  __shared__ uintx4 As[NBUF][PL][kK8][ALINE];
-  __shared__ uintx4 Bs[NBUF][PL][kK8][BLINE];
+  __shared__ uintx4 As[2][kK8][ALINE];
+  __shared__ uintx4 Bs[2][kK8][BLINE];
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -179,66 +158,44 @@ __global__ __launch_bounds__(kThreads, PL == 1 ? 3 : 2) void igemm_bf16_first(co
     }
   };
 
-  // Convert the staged chunk to bf16 terms and write it into LDS buffer `buf`.
+  // Round to bf16 and write the staged chunk into LDS buffer `buf`.
   auto stage = [&](const int buf) __attribute__((always_inline)) {
     if constexpr (GEMM) {
       // four k rows x four pixels: per pixel the four k as 8 bytes, half of a unit
+      char* line = reinterpret_cast<char*>(&Bs[buf][gkg >> 1][0]) + 8 * (gkg & 1);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        unsigned t0[PL], t1[PL];
-        terms2<PL>(breg[0][j], breg[1][j], t0);
-        terms2<PL>(breg[2][j], breg[3][j], t1);
-#pragma unroll
-        for (int pl = 0; pl < PL; ++pl) {
-          char* line = reinterpret_cast<char*>(&Bs[buf][pl][gkg >> 1][0]) + 8 * (gkg & 1);
-          *reinterpret_cast<uintx2*>(line + 16 * pos(4 * gpq + j)) = uintx2{t0[pl], t1[pl]};
-        }
-      }
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<uintx2*>(line + 16 * pos(4 * gpq + j)) =
+            uintx2{pack2(breg[0][j], breg[1][j]), pack2(breg[2][j], breg[3][j])};
     } else {
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        unsigned t[4][PL];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) terms2<PL>(breg[2 * u + (q >> 1)][2 * (q & 1)], breg[2 * u + (q >> 1)][2 * (q & 1) + 1], t[q]);
-#pragma unroll
-        for (int pl = 0; pl < PL; ++pl) Bs[buf][pl][2 * tkg + u][pos(tpx)] = uintx4{t[0][pl], t[1][pl], t[2][pl], t[3][pl]};
-      }
+      Bs[buf][2 * tkg][pos(tpx)] = uintx4{pack2(breg[0][0], breg[0][1]), pack2(breg[0][2], breg[0][3]),
+                                         pack2(breg[1][0], breg[1][1]), pack2(breg[1][2], breg[1][3])};
+      Bs[buf][2 * tkg + 1][pos(tpx)] = uintx4{pack2(breg[2][0], breg[2][1]), pack2(breg[2][2], breg[2][3]),
+                                             pack2(breg[3][0], breg[3][1]), pack2(breg[3][2], breg[3][3])};
     }
     if constexpr (AMODE == kRows) {
 #pragma unroll
-      for (int ps = 0; ps < A_PASSES; ++ps) {
-        unsigned t[4][PL];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) terms2<PL>(areg[2 * ps + (q >> 1)][2 * (q & 1)], areg[2 * ps + (q >> 1)][2 * (q & 1) + 1], t[q]);
-#pragma unroll
-        for (int pl = 0; pl < PL; ++pl) As[buf][pl][rko][pos(rrow + 64 * ps)] = uintx4{t[0][pl], t[1][pl], t[2][pl], t[3][pl]};
-      }
+      for (int ps = 0; ps < A_PASSES; ++ps)
+        As[buf][rko][pos(rrow + 64 * ps)] =
+            uintx4{pack2(areg[2 * ps][0], areg[2 * ps][1]), pack2(areg[2 * ps][2], areg[2 * ps][3]),
+                   pack2(areg[2 * ps + 1][0], areg[2 * ps + 1][1]), pack2(areg[2 * ps + 1][2], areg[2 * ps + 1][3])};
     } else if constexpr (AMODE == kCols) {
       // A_KPT k rows x four rows of the product: per row its A_KPT consecutive k
       const int k0 = A_KPT * ckg;   // first k of this thread inside the chunk
+      char* line = reinterpret_cast<char*>(&As[buf][k0 >> 3][0]) + 2 * (k0 & 7);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        unsigned t0[PL], t1[PL];
-        terms2<PL>(areg[0][j], areg[1][j], t0);
-        if constexpr (A_KPT == 4) terms2<PL>(areg[2][j], areg[3][j], t1);
-#pragma unroll
-        for (int pl = 0; pl < PL; ++pl) {
-          char* at = reinterpret_cast<char*>(&As[buf][pl][k0 >> 3][0]) + 2 * (k0 & 7) + 16 * pos(4 * ccq + j);
-          if constexpr (A_KPT == 4)
-            *reinterpret_cast<uintx2*>(at) = uintx2{t0[pl], t1[pl]};
-          else
-            *reinterpret_cast<unsigned*>(at) = t0[pl];
-        }
+        char* at = line + 16 * pos(4 * ccq + j);
+        if constexpr (A_KPT == 4)
+          *reinterpret_cast<uintx2*>(at) = uintx2{pack2(areg[0][j], areg[1][j]), pack2(areg[2][j], areg[3][j])};
+        else
+          *reinterpret_cast<unsigned*>(at) = pack2(areg[0][j], areg[1][j]);
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < A_QPT; j += 2) {
-        unsigned t[4][PL];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) terms2<PL>(areg[j + (q >> 1)][2 * (q & 1)], areg[j + (q >> 1)][2 * (q & 1) + 1], t[q]);
-#pragma unroll
-        for (int pl = 0; pl < PL; ++pl) As[buf][pl][(A_QPT * qkg + j) >> 1][pos(qrow)] = uintx4{t[0][pl], t[1][pl], t[2][pl], t[3][pl]};
-      }
+      for (int j = 0; j < A_QPT; j += 2)
+        As[buf][(A_QPT * qkg + j) >> 1][pos(qrow)] = uintx4{pack2(areg[j][0], areg[j][1]), pack2(areg[j][2], areg[j][3]),
+                                                          pack2(areg[j + 1][0], areg[j + 1][1]), pack2(areg[j + 1][2], areg[j + 1][3])};
     }
   };
 
@@ -251,28 +208,19 @@ __global__ __launch_bounds__(kThreads, PL == 1 ? 3 : 2) void igemm_bf16_first(co
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   // MFMA step kk of a chunk contracts k8-blocks 2*kk (lanes 0-31) and 2*kk + 1 (lanes 32-63): a lane's
-  // 16 bytes are its eight k of that block, the same eight for both operands.  With three terms per
-  // element the products are taken smallest first: (t2,t0) (t0,t2) (t1,t1) (t1,t0) (t0,t1) (t0,t0).
+  // 16 bytes are its eight k of that block, the same eight for both operands.
   auto multiply = [&](const int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < kK8 / 2; ++kk) {
-      bf16x8 a[MT][PL], b[NT][PL];
+      bf16x8 a[MT], b[NT];
 #pragma unroll
-      for (int pl = 0; pl < PL; ++pl) {
+      for (int x = 0; x < MT; ++x) a[x] = __builtin_bit_cast(bf16x8, As[buf][2 * kk + h][pos((wm * MT + x) * 32 + l32)]);
 #pragma unroll
-        for (int x = 0; x < MT; ++x) a[x][pl] = __builtin_bit_cast(bf16x8, As[buf][pl][2 * kk + h][pos((wm * MT + x) * 32 + l32)]);
+      for (int y = 0; y < NT; ++y) b[y] = __builtin_bit_cast(bf16x8, Bs[buf][2 * kk + h][pos((wn * NT + y) * 32 + l32)]);
 #pragma unroll
-        for (int y = 0; y < NT; ++y) b[y][pl] = __builtin_bit_cast(bf16x8, Bs[buf][pl][2 * kk + h][pos((wn * NT + y) * 32 + l32)]);
-      }
-      constexpr int kProducts = PL == 1 ? 1 : 6;
-      constexpr int ta[6] = {PL == 1 ? 0 : 2, 0, 1, 1, 0, 0}, tb[6] = {0, PL == 1 ? 0 : 2, 1, 0, 1, 0};
+      for (int x = 0; x < MT; ++x)
 #pragma unroll
-      for (int o = 0; o < kProducts; ++o)
-#pragma unroll
-        for (int x = 0; x < MT; ++x)
-#pragma unroll
-          for (int y = 0; y < NT; ++y)
-            acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x][ta[o]], b[y][tb[o]], acc[x][y], 0, 0, 0);
+        for (int y = 0; y < NT; ++y) acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[x], b[y], acc[x][y], 0, 0, 0);
     }
   };
 
@@ -280,24 +228,12 @@ __global__ __launch_bounds__(kThreads, PL == 1 ? 3 : 2) void igemm_bf16_first(co
   fetch(0);
   stage(0);
   __syncthreads();
-  if constexpr (NBUF == 2) {
-    for (int c = 0; c < chunks; ++c) {
-      const int buf = c & 1;
-      if (c + 1 < chunks) fetch(c + 1);     // in flight across this chunk's MFMAs
-      multiply(buf);
-      if (c + 1 < chunks) stage(buf ^ 1);   // the other buffer was last read before the previous barrier
-      __syncthreads();
-    }
-  } else {
-    for (int c = 0; c < chunks; ++c) {
-      if (c + 1 < chunks) fetch(c + 1);
-      multiply(0);
-      if (c + 1 < chunks) {
-        __syncthreads();                    // every wave has read the buffer
-        stage(0);
-        __syncthreads();
-      }
-    }
+  for (int c = 0; c < chunks; ++c) {
+    const int buf = c & 1;
+    if (c + 1 < chunks) fetch(c + 1);     // in flight across this chunk's MFMAs
+    multiply(buf);
+    if (c + 1 < chunks) stage(buf ^ 1);   // the other buffer was last read before the previous barrier
+    __syncthreads();
   }
 
   // ---- epilogue: accumulator register r of a 32x32 tile holds row 8*(r/4) + 4*h + r%4, column l32 ----
@@ -367,16 +303,16 @@ __global__ __launch_bounds__(kThreads, PL == 1 ? 3 : 2) void igemm_bf16_first(co
   }
 }
 
-template <int WM, int WN, int MT, int NT, int PL>
+template <int WM, int WN, int MT, int NT>
 void launch_shape(const Igemm& p, dim3 grid, int tilesM, hipStream_t st) {
   const bool gemm = p.mode == kModeGemm;
   const int amode = p.wTransStride > 0 ? kCols : (p.wRowStride > 0 ? kRows : kQuads);
-  if (gemm && amode == kRows) igemm_bf16_first<WM, WN, MT, NT, true, kRows, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
-  else if (gemm && amode == kCols) igemm_bf16_first<WM, WN, MT, NT, true, kCols, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
-  else if (gemm) igemm_bf16_first<WM, WN, MT, NT, true, kQuads, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
-  else if (amode == kRows) igemm_bf16_first<WM, WN, MT, NT, false, kRows, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
-  else if (amode == kCols) igemm_bf16_first<WM, WN, MT, NT, false, kCols, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
-  else igemm_bf16_first<WM, WN, MT, NT, false, kQuads, PL><<<grid, kThreads, 0, st>>>(p, tilesM);
+  if (gemm && amode == kRows) igemm_bf16_first<WM, WN, MT, NT, true, kRows><<<grid, kThreads, 0, st>>>(p, tilesM);
+  else if (gemm && amode == kCols) igemm_bf16_first<WM, WN, MT, NT, true, kCols><<<grid, kThreads, 0, st>>>(p, tilesM);
+  else if (gemm) igemm_bf16_first<WM, WN, MT, NT, true, kQuads><<<grid, kThreads, 0, st>>>(p, tilesM);
+  else if (amode == kRows) igemm_bf16_first<WM, WN, MT, NT, false, kRows><<<grid, kThreads, 0, st>>>(p, tilesM);
+  else if (amode == kCols) igemm_bf16_first<WM, WN, MT, NT, false, kCols><<<grid, kThreads, 0, st>>>(p, tilesM);
+  else igemm_bf16_first<WM, WN, MT, NT, false, kQuads><<<grid, kThreads, 0, st>>>(p, tilesM);
 }
 
 }  // namespace
@@ -394,17 +330,12 @@ bool bf16_first_supported(const Igemm& p, int groups, int bm) {
   return true;
 }
 
-void bf16_first_launch(const Igemm& p, int groups, int bm, int terms, hipStream_t st) {
+void bf16_first_launch(const Igemm& p, int groups, int bm, hipStream_t st) {
   const int tilesM = (p.M + 127) / 128;
   const int tilesI = p.Ipad / bm;
   const dim3 grid((unsigned)(tilesI * tilesM), (unsigned)groups);
-  if (terms == 3) {
-    if (bm == 128) launch_shape<2, 2, 2, 2, 3>(p, grid, tilesM, st);
-    else launch_shape<1, 4, 2, 1, 3>(p, grid, tilesM, st);
-  } else {
-    if (bm == 128) launch_shape<2, 2, 2, 2, 1>(p, grid, tilesM, st);
-    else launch_shape<1, 4, 2, 1, 1>(p, grid, tilesM, st);
-  }
+  if (bm == 128) launch_shape<2, 2, 2, 2>(p, grid, tilesM, st);
+  else launch_shape<1, 4, 2, 1>(p, grid, tilesM, st);
 }
 
 }  // namespace ttc

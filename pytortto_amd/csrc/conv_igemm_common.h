@@ -89,7 +89,6 @@ __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cas
 // The bf16-first kernels (conv_igemm_bf16.hip).  `supported` tells whether they take launch `p`
 // (tile rows `bm` as planned by the caller); `launch` enqueues it on the library stream.
 bool bf16_first_supported(const Igemm& p, int groups, int bm);
-// `terms`: 1 = operands rounded to bfloat16; 3 = float32 arithmetic, three bf16 terms per element.
-void bf16_first_launch(const Igemm& p, int groups, int bm, int terms, hipStream_t st);
+void bf16_first_launch(const Igemm& p, int groups, int bm, hipStream_t st);
 
 }  // namespace ttc

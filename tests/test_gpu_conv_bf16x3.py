@@ -3,7 +3,9 @@
 
 Inside the kernels every operand element becomes three bfloat16 terms that add up to it exactly and
 all products of terms except the three smallest are accumulated in float32 (what is left out stays
-below 2^-24 of a product, half an ulp of it: tests/test_bf16_round.py).  The mode therefore has to meet the float32
+below 2^-24 of a product, half an ulp of it: tests/test_bf16_round.py).  Forward and input gradient
+run that way for every geometry (the float32 kernels with another matrix step); the weight gradient
+where its reduction is long enough, and on the float32 instructions otherwise.  The mode therefore has to meet the float32
 path's own bar, and these tests hold it to exactly that: the same cases through the same checks as
 tests/test_gpu_conv.py -- allclose(rtol=1e-4, atol=1e-5) against the oracle (atol scaled by the
 tensor's magnitude for the weight / bias gradients) and no further from a float64 evaluation than
@@ -26,8 +28,8 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture
 def three_terms_everywhere():
-    """The mode, with every launch its kernels support sent to them (by default launches with fewer
-    tiles than compute units, i.e. most test shapes, stay on the float32 instructions)."""
+    """The mode, with every weight gradient its kernels support sent to them (by default those that sum
+    over fewer than 8192 pixels, i.e. most test shapes, stay on the float32 instructions)."""
     from pytortto_amd import _hip
     _hip.set_conv_math('bf16x3')
     _hip.call('tt_conv2d_bf16_first_enable', 2)
@@ -48,11 +50,13 @@ def three_terms():
         _hip.set_conv_math('f32')
 
 
-def _plan():
+def _terms_of_last_launch():
+    """bf16 terms per operand element of the matrix instructions the last forward / input-gradient
+    launch used: 0 = float32 instructions."""
     from pytortto_amd import _hip
     plan = (ctypes.c_int * 8)()
     _hip.call('tt_conv2d_last_launch', plan)
-    return list(plan)
+    return plan[7] >> 8
 
 
 @pytest.mark.parametrize('case', CONV_CASES + TILE_CASES + random_conv_cases(40, 31))
@@ -70,21 +74,23 @@ def test_conv_transpose_meets_the_float32_bar(case, three_terms_everywhere):
     _conv_transpose_checks(case)
 
 
-# (case, forward taken by the three-term kernels, input gradient taken)
+# one shape per way the kernels address their operands
 TAKEN = [
-    ((4, 64, 28, 28, 256, 1, 1, (1, 1), (0, 0), (1, 1), 1), True, True),       # 1x1: rows / columns of w in place
-    ((8, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1), True, True),      # 3x3: tap masks, repacked weights in the gradient
-    ((16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1), True, True),       # 64-row tiles
-    ((3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2), True, True),          # groups
-    ((4, 128, 28, 28, 128, 3, 3, (2, 2), (1, 1), (1, 1), 1), True, False),     # stride 2: the gradient's classes share a float32 grid
-    ((8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1), False, False),       # 49 taps: float32 instructions
+    (4, 64, 28, 28, 256, 1, 1, (1, 1), (0, 0), (1, 1), 1),       # 1x1: rows / columns of w in place
+    (8, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), (1, 1), 1),      # 3x3: tap masks, shared reductions
+    (16, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), 1),       # 64-row tiles
+    (3, 64, 6, 6, 64, 1, 1, (1, 1), (0, 0), (1, 1), 2),          # groups
+    (4, 128, 28, 28, 128, 3, 3, (2, 2), (1, 1), (1, 1), 1),      # stride 2: the gradient's classes share a grid
+    (8, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3), (1, 1), 1),         # 49 taps: 64-bit masks, dense input gradient
+    (3, 16, 14, 14, 16, 9, 9, (1, 1), (4, 4), (1, 1), 1),        # 81 taps: compared bounds
 ]
 
 
-@pytest.mark.parametrize('case,fwd_taken,dgrad_taken', TAKEN)
-def test_the_three_term_kernels_are_the_ones_that_ran(case, fwd_taken, dgrad_taken, three_terms_everywhere):
-    """-3 in the launch plan = one tile per block on the bf16-first kernels with three terms; and the
-    weight gradient's bits differ from the float32 instructions' (same sums, other rounding)."""
+@pytest.mark.parametrize('case', TAKEN)
+def test_the_three_term_kernels_are_the_ones_that_ran(case, three_terms_everywhere):
+    """The launch plan names the matrix instructions; the weight gradient's bits differ from the
+    float32 instructions' (same sums, other rounding) where its three-term kernels exist (all but the
+    64-bit-mask kernels of 32 to 63 taps)."""
     from pytortto_amd import _hip, ops
     from pytortto_amd.xparray import hiparray
     n, c, h, w_, k, r, s, st, pd, dl, g = case
@@ -92,31 +98,33 @@ def test_the_three_term_kernels_are_the_ones_that_ran(case, fwd_taken, dgrad_tak
     x = hiparray(rng.standard_normal((n, c, h, w_)).astype(np.float32))
     w = hiparray(rng.standard_normal((k, c // g, r, s)).astype(np.float32))
     y = ops.conv2d_fwd(x, w, None, st, pd, dl, g)
-    assert (_plan()[4] == -3) == fwd_taken
+    assert _terms_of_last_launch() == 3
     gy = hiparray(rng.standard_normal(y.shape).astype(np.float32))
     ops.conv2d_dgrad(gy, w, None, (h, w_), st, pd, dl, g)
-    assert (_plan()[4] == -3) == dgrad_taken
-    if r * s <= 31:
-        dw3 = ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get()
-        _hip.set_conv_math('f32')
-        dw1 = ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get()
-        _hip.set_conv_math('bf16x3')
-        assert not np.array_equal(dw3, dw1)
-        np.testing.assert_allclose(dw3, dw1, rtol=1e-4, atol=1e-5 * float(np.abs(dw1).max()))
+    assert _terms_of_last_launch() == 3
+    dw3 = ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get()
+    _hip.set_conv_math('f32')
+    ops.conv2d_fwd(x, w, None, st, pd, dl, g)
+    assert _terms_of_last_launch() == 0
+    dw1 = ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get()
+    _hip.set_conv_math('bf16x3')
+    assert np.array_equal(dw3, dw1) == (31 < r * s <= 63)
+    np.testing.assert_allclose(dw3, dw1, rtol=1e-4, atol=1e-5 * float(np.abs(dw1).max()))
 
 
-def test_by_default_only_launches_with_a_tile_per_compute_unit_are_taken(three_terms):
-    from pytortto_amd import ops
+def test_by_default_short_weight_gradient_reductions_stay_on_the_float32_instructions(three_terms):
+    from pytortto_amd import _hip, ops
     from pytortto_amd.xparray import hiparray
     rng = np.random.default_rng(5)
-    w = hiparray(rng.standard_normal((128, 128, 3, 3)).astype(np.float32))
     geo = ((1, 1), (1, 1), (1, 1), 1)
-    small = hiparray(rng.standard_normal((8, 128, 28, 28)).astype(np.float32))      # 49 tiles of 128 x 128
-    ops.conv2d_fwd(small, w, None, *geo)
-    assert _plan()[4] >= 0
-    large = hiparray(rng.standard_normal((64, 128, 28, 28)).astype(np.float32))     # 392 tiles
-    ops.conv2d_fwd(large, w, None, *geo)
-    assert _plan()[4] == -3
+    for n, same in ((8, True), (16, False)):    # 6272 and 12544 pixels to sum over
+        x = hiparray(rng.standard_normal((n, 128, 28, 28)).astype(np.float32))
+        gy = hiparray(rng.standard_normal((n, 128, 28, 28)).astype(np.float32))
+        dw3 = ops.conv2d_wgrad(x, gy, (128, 128, 3, 3), *geo).get()
+        _hip.set_conv_math('f32')
+        dw1 = ops.conv2d_wgrad(x, gy, (128, 128, 3, 3), *geo).get()
+        _hip.set_conv_math('bf16x3')
+        assert np.array_equal(dw3, dw1) == same
 
 
 def test_operands_far_from_one_keep_float32_accuracy(three_terms_everywhere):
@@ -133,7 +141,7 @@ def test_operands_far_from_one_keep_float32_accuracy(three_terms_everywhere):
     y32, xpad = oracle.convolution_forward(x, w, None, *geo)
     y64, _ = oracle.convolution_forward(x.astype(np.float64), w.astype(np.float64), None, *geo)
     y = ops.conv2d_fwd(hiparray(x), hiparray(w), None, *geo).get()
-    assert _plan()[4] == -3
+    assert _terms_of_last_launch() == 3
     scale = float(np.abs(y64).max())
     assert 1e-5 < scale < 1e-2
     assert float(np.abs(y - y64).max()) <= max(3 * float(np.abs(y32 - y64).max()), 5e-6 * scale)
@@ -160,12 +168,12 @@ def test_entry_points_for_one_call_leave_the_mode_alone():
         sfx = 'bf16x3' if how == 'call' else 'f32'
         try:
             _hip.call('tt_conv2d_fwd_' + sfx, x.ptr, w.ptr, None, y.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1)
-            taken = _plan()[4]
+            taken = _terms_of_last_launch()
             _hip.call('tt_conv2d_dgrad_' + sfx, gy.ptr, w.ptr, None, dx.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1, h, h)
             _hip.call('tt_conv2d_wgrad_' + sfx, x.ptr, gy.ptr, dw.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1, h, h)
         finally:
             _hip.set_conv_math('f32')
-        assert taken == -3
+        assert taken == 3
         assert _hip.get_conv_math() == 'f32'
         outs[how] = (y.get(), dx.get(), dw.get())
     for a, b in zip(outs['call'], outs['mode']):
