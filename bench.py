@@ -711,6 +711,35 @@ def main():
                              'stem stay on the float32 kernels\' bf16 instantiations'},
         'wgrad_tflops': round(flops_per_pass * args.steps / (bf_prof['conv_wgrad'][1] * 1e-3) / 1e12, 2),
         'kernels_ms_per_step': {k: round(v[1] / args.steps, 4) for k, v in bf_prof.items() if v[0]}}
+    progress('convolution step in float32 arithmetic on the bf16 matrix instructions (three terms)')
+    # the other optional variant, also reported separately and never part of `value`: float32
+    # arithmetic carried out on the bf16 matrix pipe (every operand element as three exact bf16
+    # terms, six products per step); it meets the float32 tolerances
+    _hip.set_conv_math('bf16x3')
+    try:
+        x3_ms, _ = timed_steps(_hip, conv_step, args.steps, args.warmup)
+        x3_prof = profiled_steps(_hip, conv_step, args.steps)
+    finally:
+        _hip.set_conv_math('f32')
+    x3_igemm_ms = x3_prof['conv_igemm_fwd'][1] + x3_prof['conv_igemm_dgrad'][1]
+    x3_igemm_tflops = igemm_flops / (x3_igemm_ms * 1e-3) / 1e12
+    x3_peak = PEAK_BF16_MFMA_TFLOPS / 6.0
+    bf16x3_variant = {
+        'metric': 'conv fwd+bwd TFLOP/s, float32 arithmetic on bf16 MFMA (forward, input gradient, weight gradient)',
+        'value': round(3 * flops_per_pass / (x3_ms * 1e-3) / 1e12, 2), 'unit': 'TFLOP/s',
+        'ms_per_step': round(x3_ms, 3), 'speedup_over_f32_step': round(conv_ms / x3_ms, 3),
+        'dtype': 'f32 operands as three exact bf16 terms each, six bf16 MFMAs per product step, f32 accumulation',
+        'error_bound': 'the float32 tolerances (rtol 1e-4 / atol 1e-5 against the oracle): the three products of terms left '
+                       'out stay below 2^-24 of a product',
+        'roofline': {'bound': 'mfma', 'kernel': 'igemm_bf16x3 (Conv2d forward + input gradient)',
+                     'achieved': round(x3_igemm_tflops, 2), 'peak': round(x3_peak, 1), 'unit': 'TFLOP/s',
+                     'frac': round(x3_igemm_tflops / x3_peak, 4), 'traffic': None,
+                     'speedup_over_f32_kernel': round((ms_fwd + ms_dg) / x3_igemm_ms, 2),
+                     'note': 'peak = the bf16 MFMA peak divided by the six matrix instructions a product step takes; '
+                             'achieved = useful float32 FLOPs (2*N*K*C*R*S*P*Q) per second.  The kernels are bound by the '
+                             'vector instructions that form the terms, not by the matrix pipe'},
+        'wgrad_tflops': round(flops_per_pass * args.steps / (x3_prof['conv_wgrad'][1] * 1e-3) / 1e12, 2),
+        'kernels_ms_per_step': {k: round(v[1] / args.steps, 4) for k, v in x3_prof.items() if v[0]}}
     del layers
     call('tt_empty_cache')
 
@@ -794,6 +823,14 @@ def main():
             _hip.set_conv_math('f32')
         model['with_bf16_conv_math'] = {'value': round(b_ips, 1), 'unit': 'images/s', 'ms_per_step': round(b_wall, 2),
                                         'loss_first_last': [round(b_losses[0], 4), round(b_losses[-1], 4)]}
+        call('tt_empty_cache')
+        _hip.set_conv_math('bf16x3')   # float32 arithmetic on the bf16 matrix instructions: same tolerances as fp32
+        try:
+            t_ips, t_ms, t_wall, t_losses = resnet50_train_step(_hip, max(3, args.steps // 2), 2)
+        finally:
+            _hip.set_conv_math('f32')
+        model['with_bf16x3_conv_math'] = {'value': round(t_ips, 1), 'unit': 'images/s', 'ms_per_step': round(t_wall, 2),
+                                          'loss_first_last': [round(t_losses[0], 4), round(t_losses[-1], 4)]}
         call('tt_empty_cache')
 
     progress('PreAct-ResNet-18 and DCGAN stacks')
@@ -892,6 +929,7 @@ def main():
                               'roofline_tflops = min(157.3, AI * 8 TB/s), AI = F / (4 * (|x| + |w| + |y|))',
                       'rows': layer_rows},
         'conv_bf16_variant': bf16_variant,
+        'conv_bf16x3_variant': bf16x3_variant,
         'cpu_baseline': cpu_conv,
         'single_layer_config': c1_gpu,
         'bn': {'metric': 'BatchNorm2d training fwd+bwd GB/s', 'value': round(bn_gbs, 1), 'unit': 'GB/s',
