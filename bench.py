@@ -725,7 +725,7 @@ def main():
     x3_igemm_tflops = igemm_flops / (x3_igemm_ms * 1e-3) / 1e12
     x3_peak = PEAK_BF16_MFMA_TFLOPS / 6.0
     bf16x3_variant = {
-        'metric': 'conv fwd+bwd TFLOP/s, float32 arithmetic on bf16 MFMA (forward, input gradient, weight gradient)',
+        'metric': 'conv fwd+bwd TFLOP/s, float32 arithmetic on bf16 MFMA (forward and input gradient; weight gradient on fp32 MFMA)',
         'value': round(3 * flops_per_pass / (x3_ms * 1e-3) / 1e12, 2), 'unit': 'TFLOP/s',
         'ms_per_step': round(x3_ms, 3), 'speedup_over_f32_step': round(conv_ms / x3_ms, 3),
         'dtype': 'f32 operands as three exact bf16 terms each, six bf16 MFMAs per product step, f32 accumulation',
@@ -737,7 +737,8 @@ def main():
                      'speedup_over_f32_kernel': round((ms_fwd + ms_dg) / x3_igemm_ms, 2),
                      'note': 'peak = the bf16 MFMA peak divided by the six matrix instructions a product step takes; '
                              'achieved = useful float32 FLOPs (2*N*K*C*R*S*P*Q) per second.  The kernels are bound by the '
-                             'vector instructions that form the terms, not by the matrix pipe'},
+                             'latencies of a 16-deep chunk (global load, LDS, barrier), not by the matrix pipe: with the terms '
+                             'left unformed or five of the six products left out (throw-away builds) they take 65-80 % as long'},
         'wgrad_tflops': round(flops_per_pass * args.steps / (x3_prof['conv_wgrad'][1] * 1e-3) / 1e12, 2),
         'kernels_ms_per_step': {k: round(v[1] / args.steps, 4) for k, v in x3_prof.items() if v[0]}}
     del layers

@@ -113,9 +113,8 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
  * no more than rounding the product to float32 once.  Results meet the same tolerances as TT_CONV_MATH_F32 (they differ from it as two
  * float32 summation orders do); non-finite operands and magnitudes above 3.38e38 (which round to a
  * bf16 infinity) give NaN where float32 would give an infinity.  Forward and input gradient run
- * that way for every geometry; weight gradients it does not pay for (fewer than 8192 pixels to sum
- * over, 64-row tiles of kernels larger than 1x1, kernels of 32 to 63 taps) run on the float32
- * instructions.
+ * that way for every geometry; the weight gradient keeps the float32 instructions (its loop is bound
+ * by streaming x and dy through LDS, and three-term variants of it measured no faster).
  * The modes apply to tt_conv2d_fwd_f32,
  * tt_conv2d_dgrad_f32 and tt_conv2d_wgrad_f32.  The setting is process-wide and applies to
  * later calls of every caller; the *_bf16 and *_bf16x3 entry points below select a mode per call
@@ -123,10 +122,10 @@ int tt_probe_hbm_f32(size_t bytes, double* read_gbs, double* copy_gbs);
 enum { TT_CONV_MATH_F32 = 0, TT_CONV_MATH_BF16 = 1, TT_CONV_MATH_BF16X3 = 2 };
 int tt_set_conv_math(int mode);
 int tt_get_conv_math(int* mode);   /* host pointer */
-/* The same three passes with bf16 (*_bf16) or three-term (*_bf16x3) matrix arithmetic for one call,
- * whatever the process-wide mode is (arguments as tt_conv2d_fwd_f32 / tt_conv2d_dgrad_f32 /
- * tt_conv2d_wgrad_f32 below; tensors are float32): for callers that must not change what other
- * callers of the library compute. */
+/* The same passes with bf16 (*_bf16) or three-term (*_bf16x3: forward and input gradient) matrix
+ * arithmetic for one call, whatever the process-wide mode is (arguments as tt_conv2d_fwd_f32 /
+ * tt_conv2d_dgrad_f32 / tt_conv2d_wgrad_f32 below; tensors are float32): for callers that must not
+ * change what other callers of the library compute. */
 int tt_conv2d_fwd_bf16(const float* x, const float* w, const float* bias, float* y,
                        int N, int C, int H, int W, int K, int R, int S,
                        int sh, int sw, int ph, int pw, int dh, int dw, int groups);
@@ -142,9 +141,7 @@ int tt_conv2d_fwd_bf16x3(const float* x, const float* w, const float* bias, floa
 int tt_conv2d_dgrad_bf16x3(const float* dy, const float* w, const float* bias, float* dx,
                            int N, int C, int Hx, int Wx, int K, int R, int S,
                            int sh, int sw, int ph, int pw, int dh, int dw, int groups, int P, int Q);
-int tt_conv2d_wgrad_bf16x3(const float* x, const float* dy, float* dw,
-                           int N, int C, int H, int W, int K, int R, int S,
-                           int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q);
+
 
 /* Tuning threshold of tt_conv2d_dgrad_f32 for strided layers with very few input channels (the
  * ResNet stem, the output layer of a transposed generator), no counterpart in the reference.
@@ -254,8 +251,7 @@ int tt_conv2d_last_launch(int* plan8);
  * most 1024 (1, the default) or whenever those kernels support the geometry (2: small test shapes);
  * 0 keeps every launch on the float32 kernels' bf16 instantiations, which also serve the launches
  * the former do not take.  Both compute the same thing: the convolution of
- * the bf16-rounded operands in float32.  With TT_CONV_MATH_BF16X3, 2 sends every weight gradient
- * the three-term kernels support to them, whatever the size rule says. */
+ * the bf16-rounded operands in float32. */
 int tt_conv2d_bf16_first_enable(int on);
 int tt_conv2d_last_wgrad_launch(int* plan4);
 int tt_conv2d_wgrad_force_occupancy(int blocks);

@@ -46,7 +46,6 @@ PROTOTYPES = {
     'tt_conv2d_wgrad_bf16': [_P, _P, _P] + [_I] * 16,
     'tt_conv2d_fwd_bf16x3': [_P, _P, _P, _P] + [_I] * 14,
     'tt_conv2d_dgrad_bf16x3': [_P, _P, _P, _P] + [_I] * 16,
-    'tt_conv2d_wgrad_bf16x3': [_P, _P, _P] + [_I] * 16,
     'tt_conv2d_check_tables_fwd_f32': [_I] * 14,
     'tt_conv2d_check_tables_dgrad_f32': [_I] * 16,
     'tt_conv2d_check_tables_wgrad_f32': [_I] * 16,

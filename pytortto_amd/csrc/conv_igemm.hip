@@ -1116,12 +1116,6 @@ int g_last_launch[8] = {};
 bool g_bf16_first = true;
 bool g_bf16_first_always = false;   // tests: also where the tile-count rule would keep the other kernels
 
-}  // namespace
-namespace tt {
-bool conv_bf16_kernels_forced() { return g_bf16_first_always; }
-}
-namespace {
-
 int launch_igemm(Igemm& p, int groups, TileChoice t, int prof_id, floatx4* sk_partial) {
   tt::ProfScope prof(prof_id);
   p.tilesI = p.Ipad / t.bm;

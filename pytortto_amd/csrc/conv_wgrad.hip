@@ -99,18 +99,6 @@ __device__ __forceinline__ unsigned pack2(float lo, float hi) {   // two floats 
   const bf16x2 v = {(__bf16)lo, (__bf16)hi};
   return __builtin_bit_cast(unsigned, v);
 }
-// Two float32 values as PL pairs of bfloat16: rounded (PL = 1), or as three terms that add up to them
-// exactly, each the bf16 nearest to what the terms before it leave (PL = 3; the differences are exact).
-template <int PL>
-__device__ __forceinline__ void terms2(float lo, float hi, unsigned (&t)[PL]) {
-  t[0] = pack2(lo, hi);
-  if constexpr (PL == 3) {
-    const float l1 = lo - __uint_as_float(t[0] << 16), h1 = hi - __uint_as_float(t[0] & 0xffff0000u);
-    t[1] = pack2(l1, h1);
-    const float l2 = l1 - __uint_as_float(t[1] << 16), h2 = h1 - __uint_as_float(t[1] & 0xffff0000u);
-    t[2] = pack2(l2, h2);
-  }
-}
 __device__ __forceinline__ int pos16(int i) { return i + (i >> 4); }   // unit of row i in a bf16 LDS line
 // The value the next lane holds (lanes 0, 2 of every quad get lanes 1, 3; odd lanes get their own).
 __device__ __forceinline__ float next_lane(float v) {
@@ -123,16 +111,10 @@ __device__ __forceinline__ float next_lane(float v) {
 // (thread = (row group of 32, pixel quad) instead of (row group of 8, pixel)).  VA needs P*Q to be
 // a multiple of 4 so that a quad never straddles two images, VB in addition a 1x1, stride-1,
 // unpadded layer, where x is indexed by the output pixel like dy and has no padding to mask.
-// PL: 0 = float32 matrix instructions.  1 = the optional bf16 variant (tt_set_conv_math): operands
-// rounded to bfloat16 on their way into LDS, v_mfma_f32_32x32x16_bf16, float32 accumulation.  3 = float32
-// arithmetic on the bf16 matrix pipe: every operand element enters LDS as three bf16 terms that add up
-// to it exactly and the six products of terms that matter are accumulated (one LDS buffer, two
-// barriers per chunk).
-template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB, int PL, bool WIDE = false>
+// BF: the optional bf16 variant (tt_set_conv_math): operands rounded to bfloat16 after the LDS
+// read, v_mfma_f32_32x32x16_bf16, float32 accumulation.
+template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB, bool BF, bool WIDE = false>
 __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
-  constexpr bool BF = PL > 0;
-  constexpr int PLN = PL > 0 ? PL : 1;
-  static_assert(PL == 0 || PL == 1 || PL == 3, "bf16 terms per operand element");
   static_assert(WM * WN == 4, "four waves per block");
   static_assert(BUF || (!VA && !VB), "vector fetches belong to the buffer path");
   static_assert(!WIDE || (BUF && !VB), "64-bit tap masks belong to the buffer path of kernels larger than 1x1");
@@ -145,9 +127,8 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   // sixteen, lines 12 or 4 units past a multiple of sixteen so that the four lines of a chunk spread
   // over the banks): half the LDS bytes and no conversion next to the matrix instructions.
   constexpr int ALINE = BM == 128 ? 140 : 68, BLINE = BN == 128 ? 140 : 68;
-  constexpr int kUnits16 = PL == 3 ? 3 : 2;   // [buffer] for one term, [term] for three
-  constexpr size_t kBytesA = BF ? sizeof(uintx4) * kUnits16 * 4 * ALINE : sizeof(float) * 2 * BM * kLd;
-  constexpr size_t kBytesB = BF ? sizeof(uintx4) * kUnits16 * 4 * BLINE : sizeof(float) * 2 * BN * kLd;
+  constexpr size_t kBytesA = BF ? sizeof(uintx4) * 2 * 4 * ALINE : sizeof(float) * 2 * BM * kLd;
+  constexpr size_t kBytesB = BF ? sizeof(uintx4) * 2 * 4 * BLINE : sizeof(float) * 2 * BN * kLd;
   __shared__ __attribute__((aligned(16))) char lds[kBytesA + kBytesB];
   char* const ldsA = lds;
   char* const ldsB = lds + kBytesA;
@@ -316,50 +297,32 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
   // outside the image must be exactly zero: AND with an all-ones / all-zeros word.
   auto store_step = [&](int buf, int li, const int set = 0) __attribute__((always_inline)) {
     if constexpr (BF) {
-      // Convert to bf16 terms and write pixel-major units.  Vector fetches hold four consecutive pixels
-      // of a row: 8 bytes, half a unit.  Scalar fetches hold one pixel per lane: every even lane takes
-      // its neighbour's value too and writes the pair.  (Masks of the compare path apply first.)
+      // Round to bf16 and write pixel-major units.  Vector fetches hold four consecutive pixels of a
+      // row: 8 bytes, half a unit.  Scalar fetches hold one pixel per lane: every even lane takes its
+      // neighbour's value too and writes the pair.  (Masks of the compare path apply first.)
       if (li < A_ROWS) {
         if constexpr (VA) {
           const floatx4 v = aregv[set][li];
-          unsigned t0[PLN], t1[PLN];
-          terms2<PLN>(v[0], v[1], t0);
-          terms2<PLN>(v[2], v[3], t1);
-#pragma unroll
-          for (int pl = 0; pl < PLN; ++pl)
-            *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&As16[PL == 3 ? pl : buf][qpx >> 1][pos16(rgq + 32 * li)]) + 8 * (qpx & 1)) =
-                uintx2{t0[pl], t1[pl]};
+          *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&As16[buf][qpx >> 1][pos16(rgq + 32 * li)]) + 8 * (qpx & 1)) =
+              uintx2{pack2(v[0], v[1]), pack2(v[2], v[3])};
         } else {
           const float v = BUF ? areg[set][li] : __int_as_float(__float_as_int(areg[set][li]) & amask[set]);
-          unsigned pair[PLN];
-          terms2<PLN>(v, next_lane(v), pair);
-          if ((px & 1) == 0) {
-#pragma unroll
-            for (int pl = 0; pl < PLN; ++pl)
-              *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&As16[PL == 3 ? pl : buf][px >> 3][pos16(rg + 8 * li)]) + 2 * (px & 7)) = pair[pl];
-          }
+          const unsigned pair = pack2(v, next_lane(v));
+          if ((px & 1) == 0)
+            *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&As16[buf][px >> 3][pos16(rg + 8 * li)]) + 2 * (px & 7)) = pair;
         }
       } else {
         const int t = li - A_ROWS;
         if constexpr (VB) {
           const floatx4 v = bregv[set][t];
-          unsigned t0[PLN], t1[PLN];
-          terms2<PLN>(v[0], v[1], t0);
-          terms2<PLN>(v[2], v[3], t1);
-#pragma unroll
-          for (int pl = 0; pl < PLN; ++pl)
-            *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&Bs16[PL == 3 ? pl : buf][qpx >> 1][pos16(rgq + 32 * t)]) + 8 * (qpx & 1)) =
-                uintx2{t0[pl], t1[pl]};
+          *reinterpret_cast<uintx2*>(reinterpret_cast<char*>(&Bs16[buf][qpx >> 1][pos16(rgq + 32 * t)]) + 8 * (qpx & 1)) =
+              uintx2{pack2(v[0], v[1]), pack2(v[2], v[3])};
         } else {
           const int bmask = ((int)(bok[set] << (31 - t))) >> 31;
           const float v = BUF ? breg[set][t] : __int_as_float(__float_as_int(breg[set][t]) & bmask);
-          unsigned pair[PLN];
-          terms2<PLN>(v, next_lane(v), pair);
-          if ((px & 1) == 0) {
-#pragma unroll
-            for (int pl = 0; pl < PLN; ++pl)
-              *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&Bs16[PL == 3 ? pl : buf][px >> 3][pos16(rg + 8 * t)]) + 2 * (px & 7)) = pair[pl];
-          }
+          const unsigned pair = pack2(v, next_lane(v));
+          if ((px & 1) == 0)
+            *reinterpret_cast<unsigned*>(reinterpret_cast<char*>(&Bs16[buf][px >> 3][pos16(rg + 8 * t)]) + 2 * (px & 7)) = pair;
         }
       }
       return;
@@ -428,32 +391,22 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        bf16x8 a[MT][PLN], b[NT][PLN];
+        bf16x8 a[MT], b[NT];
 #pragma unroll
-        for (int pl = 0; pl < PLN; ++pl) {
+        for (int xx = 0; xx < MT; ++xx)
+          a[xx] = __builtin_bit_cast(bf16x8, As16[buf][2 * t + h][pos16((wm * MT + xx) * 32 + l32)]);
 #pragma unroll
-          for (int xx = 0; xx < MT; ++xx)
-            a[xx][pl] = __builtin_bit_cast(bf16x8, As16[PL == 3 ? pl : buf][2 * t + h][pos16((wm * MT + xx) * 32 + l32)]);
+        for (int yy = 0; yy < NT; ++yy)
+          b[yy] = __builtin_bit_cast(bf16x8, Bs16[buf][2 * t + h][pos16((wn * NT + yy) * 32 + l32)]);
+#pragma unroll
+        for (int xx = 0; xx < MT; ++xx)
 #pragma unroll
           for (int yy = 0; yy < NT; ++yy)
-            b[yy][pl] = __builtin_bit_cast(bf16x8, Bs16[PL == 3 ? pl : buf][2 * t + h][pos16((wn * NT + yy) * 32 + l32)]);
-        }
-        // three terms: the products smallest first, (t2,t0) (t0,t2) (t1,t1) (t1,t0) (t0,t1) (t0,t0)
-        constexpr int kProducts = PL == 3 ? 6 : 1;
-        constexpr int ta[6] = {PL == 3 ? 2 : 0, 0, 1, 1, 0, 0}, tb[6] = {0, PL == 3 ? 2 : 0, 1, 0, 1, 0};
-#pragma unroll
-        for (int o = 0; o < kProducts; ++o)
-#pragma unroll
-          for (int xx = 0; xx < MT; ++xx)
-#pragma unroll
-            for (int yy = 0; yy < NT; ++yy)
-              acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[xx][ta[o]], b[yy][tb[o]], acc[xx][yy], 0, 0, 0);
+            acc[xx][yy] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[xx], b[yy], acc[xx][yy], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       // the chunk after this one was fetched during the previous chunk: it has had a whole chunk's
-      // time to arrive and goes to the other LDS buffer now (three terms: to the one buffer, once
-      // every wave has read it)
-      if constexpr (PL == 3) __syncthreads();
+      // time to arrive and goes to the other LDS buffer now
 #pragma unroll
       for (int li = 0; li < L; ++li) store_step(buf ^ 1, li, buf ^ 1);
       __syncthreads();
@@ -624,24 +577,20 @@ __device__ __forceinline__ void wgrad_body(const Wgrad& p) {
 
 template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_f32(const Wgrad p) {
-  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, 0>(p);
+  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, false>(p);
 }
 template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_bf16(const Wgrad p) {
-  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, 1>(p);
-}
-template <int WM, int WN, int MT, int NT, bool BUF, bool VA, bool VB>
-__global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_bf16x3(const Wgrad p) {
-  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, 3>(p);
+  wgrad_body<WM, WN, MT, NT, BUF, VA, VB, true>(p);
 }
 // kernels of 32 .. 63 taps: buffer path with 64-bit tap masks
 template <int WM, int WN, int MT, int NT, bool VA>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_wide_f32(const Wgrad p) {
-  wgrad_body<WM, WN, MT, NT, true, VA, false, 0, true>(p);
+  wgrad_body<WM, WN, MT, NT, true, VA, false, false, true>(p);
 }
 template <int WM, int WN, int MT, int NT, bool VA>
 __global__ __launch_bounds__(kThreads, 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void wgrad_wide_bf16(const Wgrad p) {
-  wgrad_body<WM, WN, MT, NT, true, VA, false, 1, true>(p);
+  wgrad_body<WM, WN, MT, NT, true, VA, false, true, true>(p);
 }
 
 // dw[e] = sum over splits of partial[s][e] in float64.  A block covers 64 float4 columns with
@@ -898,25 +847,19 @@ int cached_pixtab(const char* fn, const PixGeom& g, bool wide, bool host_only, c
 
 typedef void (*WgradKernel)(const Wgrad);
 template <int WM, int WN, int MT, int NT>
-WgradKernel pick_wgrad(int math, bool buf, bool va, bool vb, bool wide) {
+WgradKernel pick_wgrad(bool buf, bool va, bool vb, bool wide) {
   if (wide) {   // implies buf and not vb
-    const bool bf = math == TT_CONV_MATH_BF16;
+    const bool bf = tt::conv_math() == TT_CONV_MATH_BF16;
     if (bf && va) return wgrad_wide_bf16<WM, WN, MT, NT, true>;
     if (bf) return wgrad_wide_bf16<WM, WN, MT, NT, false>;
     if (va) return wgrad_wide_f32<WM, WN, MT, NT, true>;
     return wgrad_wide_f32<WM, WN, MT, NT, false>;
   }
-  if (math == TT_CONV_MATH_BF16) {
+  if (tt::conv_math() == TT_CONV_MATH_BF16) {
     if (buf && va && vb) return wgrad_bf16<WM, WN, MT, NT, true, true, true>;
     if (buf && va) return wgrad_bf16<WM, WN, MT, NT, true, true, false>;
     if (buf) return wgrad_bf16<WM, WN, MT, NT, true, false, false>;
     return wgrad_bf16<WM, WN, MT, NT, false, false, false>;
-  }
-  if (math == TT_CONV_MATH_BF16X3) {   // (the 32 .. 63-tap kernels above stay on float32 instructions)
-    if (buf && va && vb) return wgrad_bf16x3<WM, WN, MT, NT, true, true, true>;
-    if (buf && va) return wgrad_bf16x3<WM, WN, MT, NT, true, true, false>;
-    if (buf) return wgrad_bf16x3<WM, WN, MT, NT, true, false, false>;
-    return wgrad_bf16x3<WM, WN, MT, NT, false, false, false>;
   }
   if (buf && va && vb) return wgrad_f32<WM, WN, MT, NT, true, true, true>;
   if (buf && va) return wgrad_f32<WM, WN, MT, NT, true, true, false>;
@@ -1090,18 +1033,11 @@ static int conv2d_wgrad(const float* x, const float* dy, float* dw, int N, int C
     // 16-byte fetches along the reduction: whole pixel quads inside one image, aligned tensors
     const bool va = buf && (P * Q) % 4 == 0 && ((uintptr_t)p.dy & 15) == 0;
     const bool vb = va && R == 1 && S == 1 && sh == 1 && sw == 1 && ph == 0 && pw == 0 && ((uintptr_t)p.x & 15) == 0;
-    // float32 arithmetic on the bf16 pipe (three terms per element) pays where the reduction is long
-    // enough to amortise its two barriers per chunk (measured on the ResNet-50 shapes at batch 64:
-    // 1.05-1.25 times faster from 12544 pixels on, slower at 3136 and for 64-row tiles of 3x3
-    // layers); other launches of that mode stay on the float32 instructions.
-    int math = tt::conv_math();
-    if (math == TT_CONV_MATH_BF16X3 && !tt::conv_bf16_kernels_forced() && (p.M < 8192 || (bm == 64 && R * S > 1)))
-      math = TT_CONV_MATH_F32;
     WgradKernel kernel;
-    if (bm == 128 && bn == 128) kernel = pick_wgrad<2, 2, 2, 2>(math, buf, va, vb, wide);
-    else if (bm == 64 && bn == 128) kernel = pick_wgrad<2, 2, 1, 2>(math, buf, va, vb, wide);
-    else if (bm == 128 && bn == 64) kernel = pick_wgrad<2, 2, 2, 1>(math, buf, va, vb, wide);
-    else kernel = pick_wgrad<2, 2, 1, 1>(math, buf, va, vb, wide);
+    if (bm == 128 && bn == 128) kernel = pick_wgrad<2, 2, 2, 2>(buf, va, vb, wide);
+    else if (bm == 64 && bn == 128) kernel = pick_wgrad<2, 2, 1, 2>(buf, va, vb, wide);
+    else if (bm == 128 && bn == 64) kernel = pick_wgrad<2, 2, 2, 1>(buf, va, vb, wide);
+    else kernel = pick_wgrad<2, 2, 1, 1>(buf, va, vb, wide);
     if (ws == nullptr && slots > 1) {   // first run: now the kernel is known, and with it what the device holds of it
       fused = fuse_shape && tiles * r.splits <= resident_blocks(kernel);
       if (tt::workspace(fused ? fuse_bytes : sizeof(float) * elems * slots, &ws)) return -1;

@@ -349,13 +349,6 @@ int tt_conv2d_dgrad_bf16x3(const float* dy, const float* w, const float* bias, f
   return tt_conv2d_dgrad_f32(dy, w, bias, dx, N, C, Hx, Wx, K, R, S_, sh, sw, ph, pw, dh, dw, groups, P, Q);
 }
 
-int tt_conv2d_wgrad_bf16x3(const float* x, const float* dy, float* dw, int N, int C, int H, int W, int K, int R, int S_,
-                           int sh, int sw, int ph, int pw, int dh, int dw_, int groups, int P, int Q) {
-  TT_API_LOCK();
-  ScopedMath mode(TT_CONV_MATH_BF16X3);
-  return tt_conv2d_wgrad_f32(x, dy, dw, N, C, H, W, K, R, S_, sh, sw, ph, pw, dh, dw_, groups, P, Q);
-}
-
 int tt_sync(void) {
   TT_REQUIRE_INIT();
   TT_HIP(hipStreamSynchronize(S().stream));

@@ -61,9 +61,6 @@ constexpr int kWave = 64;
 
 // Matrix arithmetic of the convolution kernels: TT_CONV_MATH_F32, _BF16 or _BF16X3 (tt_set_conv_math).
 int conv_math();
-// Tests (tt_conv2d_bf16_first_enable(2)): every launch the bf16 kernels support goes to them, whatever
-// the size rules of the bf16 modes say.
-bool conv_bf16_kernels_forced();
 
 inline bool fits_i32(long long elems) { return elems >= 0 && elems < 2147483647LL; }
 

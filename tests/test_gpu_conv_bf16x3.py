@@ -5,7 +5,7 @@ Inside the kernels every operand element becomes three bfloat16 terms that add u
 all products of terms except the three smallest are accumulated in float32 (what is left out stays
 below 2^-24 of a product, half an ulp of it: tests/test_bf16_round.py).  Forward and input gradient
 run that way for every geometry (the float32 kernels with another matrix step); the weight gradient
-where its reduction is long enough, and on the float32 instructions otherwise.  The mode therefore has to meet the float32
+keeps the float32 instructions and must not change with the mode.  The mode therefore has to meet the float32
 path's own bar, and these tests hold it to exactly that: the same cases through the same checks as
 tests/test_gpu_conv.py -- allclose(rtol=1e-4, atol=1e-5) against the oracle (atol scaled by the
 tensor's magnitude for the weight / bias gradients) and no further from a float64 evaluation than
@@ -24,20 +24,6 @@ from tests.test_gpu_conv import test_conv_transpose_forward_backward as _conv_tr
 from tests.test_gpu_full_size_shapes import test_shape_at_full_batch_properties as _full_size_checks
 
 pytestmark = pytest.mark.gpu
-
-
-@pytest.fixture
-def three_terms_everywhere():
-    """The mode, with every weight gradient its kernels support sent to them (by default those that sum
-    over fewer than 8192 pixels, i.e. most test shapes, stay on the float32 instructions)."""
-    from pytortto_amd import _hip
-    _hip.set_conv_math('bf16x3')
-    _hip.call('tt_conv2d_bf16_first_enable', 2)
-    try:
-        yield
-    finally:
-        _hip.call('tt_conv2d_bf16_first_enable', 1)
-        _hip.set_conv_math('f32')
 
 
 @pytest.fixture
@@ -60,17 +46,17 @@ def _terms_of_last_launch():
 
 
 @pytest.mark.parametrize('case', CONV_CASES + TILE_CASES + random_conv_cases(40, 31))
-def test_conv_meets_the_float32_bar(case, three_terms_everywhere):
+def test_conv_meets_the_float32_bar(case, three_terms):
     _run_conv(case)
 
 
 @pytest.mark.parametrize('case', TILE_CASES[:16])
-def test_conv_without_bias_meets_the_float32_bar(case, three_terms_everywhere):
+def test_conv_without_bias_meets_the_float32_bar(case, three_terms):
     _run_conv(case, seed=9, bias=False)
 
 
 @pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES + random_convt_cases(12, 17))
-def test_conv_transpose_meets_the_float32_bar(case, three_terms_everywhere):
+def test_conv_transpose_meets_the_float32_bar(case, three_terms):
     _conv_transpose_checks(case)
 
 
@@ -87,10 +73,8 @@ TAKEN = [
 
 
 @pytest.mark.parametrize('case', TAKEN)
-def test_the_three_term_kernels_are_the_ones_that_ran(case, three_terms_everywhere):
-    """The launch plan names the matrix instructions; the weight gradient's bits differ from the
-    float32 instructions' (same sums, other rounding) where its three-term kernels exist (all but the
-    64-bit-mask kernels of 32 to 63 taps)."""
+def test_the_three_term_kernels_are_the_ones_that_ran(case, three_terms):
+    """The launch plan names the matrix instructions; the weight gradient does not depend on the mode."""
     from pytortto_amd import _hip, ops
     from pytortto_amd.xparray import hiparray
     n, c, h, w_, k, r, s, st, pd, dl, g = case
@@ -108,26 +92,10 @@ def test_the_three_term_kernels_are_the_ones_that_ran(case, three_terms_everywhe
     assert _terms_of_last_launch() == 0
     dw1 = ops.conv2d_wgrad(x, gy, w.shape, st, pd, dl, g).get()
     _hip.set_conv_math('bf16x3')
-    assert np.array_equal(dw3, dw1) == (31 < r * s <= 63)
-    np.testing.assert_allclose(dw3, dw1, rtol=1e-4, atol=1e-5 * float(np.abs(dw1).max()))
+    np.testing.assert_array_equal(dw3, dw1)
 
 
-def test_by_default_short_weight_gradient_reductions_stay_on_the_float32_instructions(three_terms):
-    from pytortto_amd import _hip, ops
-    from pytortto_amd.xparray import hiparray
-    rng = np.random.default_rng(5)
-    geo = ((1, 1), (1, 1), (1, 1), 1)
-    for n, same in ((8, True), (16, False)):    # 6272 and 12544 pixels to sum over
-        x = hiparray(rng.standard_normal((n, 128, 28, 28)).astype(np.float32))
-        gy = hiparray(rng.standard_normal((n, 128, 28, 28)).astype(np.float32))
-        dw3 = ops.conv2d_wgrad(x, gy, (128, 128, 3, 3), *geo).get()
-        _hip.set_conv_math('f32')
-        dw1 = ops.conv2d_wgrad(x, gy, (128, 128, 3, 3), *geo).get()
-        _hip.set_conv_math('bf16x3')
-        assert np.array_equal(dw3, dw1) == same
-
-
-def test_operands_far_from_one_keep_float32_accuracy(three_terms_everywhere):
+def test_operands_far_from_one_keep_float32_accuracy(three_terms):
     """bfloat16 has float32's exponent range: operands of 1e-20 and 1e+15 need no scaling (a split into
     float16 terms would lose them), and zeros stay zeros."""
     from pytortto_amd import ops
@@ -170,7 +138,7 @@ def test_entry_points_for_one_call_leave_the_mode_alone():
             _hip.call('tt_conv2d_fwd_' + sfx, x.ptr, w.ptr, None, y.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1)
             taken = _terms_of_last_launch()
             _hip.call('tt_conv2d_dgrad_' + sfx, gy.ptr, w.ptr, None, dx.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1, h, h)
-            _hip.call('tt_conv2d_wgrad_' + sfx, x.ptr, gy.ptr, dw.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1, h, h)
+            _hip.call('tt_conv2d_wgrad_f32', x.ptr, gy.ptr, dw.ptr, n, c, h, h, k, 3, 3, 1, 1, 1, 1, 1, 1, 1, h, h)
         finally:
             _hip.set_conv_math('f32')
         assert taken == 3
