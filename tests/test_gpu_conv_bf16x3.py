@@ -19,7 +19,7 @@ import pytest
 import oracle
 from bench import RESNET50_CONVS
 from tests.cases import CONV_CASES, CONVT_CASES, random_conv_cases, random_convt_cases
-from tests.test_gpu_conv import CONVT_TILE_CASES, TILE_CASES, _check, _run_conv
+from tests.test_gpu_conv import CONVT_TILE_CASES, LARGE_IMAGE_CASES, TILE_CASES, _check, _run_conv
 from tests.test_gpu_conv import test_conv_transpose_forward_backward as _conv_transpose_checks
 from tests.test_gpu_full_size_shapes import test_shape_at_full_batch_properties as _full_size_checks
 
@@ -53,6 +53,12 @@ def test_conv_meets_the_float32_bar(case, three_terms):
 @pytest.mark.parametrize('case', TILE_CASES[:16])
 def test_conv_without_bias_meets_the_float32_bar(case, three_terms):
     _run_conv(case, seed=9, bias=False)
+
+
+@pytest.mark.parametrize('case', LARGE_IMAGE_CASES)
+def test_conv_large_images_meet_the_float32_bar(case, three_terms):
+    """Images too large for 32-bit offsets: 64-bit addresses with compared bounds, also in this arithmetic."""
+    _run_conv(case, seed=3)
 
 
 @pytest.mark.parametrize('case', CONVT_CASES + CONVT_TILE_CASES + random_convt_cases(12, 17))
