@@ -737,8 +737,9 @@ def main():
                      'speedup_over_f32_kernel': round((ms_fwd + ms_dg) / x3_igemm_ms, 2),
                      'note': 'peak = the bf16 MFMA peak divided by the six matrix instructions a product step takes; '
                              'achieved = useful float32 FLOPs (2*N*K*C*R*S*P*Q) per second.  The kernels are bound by the '
-                             'latencies of a 16-deep chunk (global load, LDS, barrier), not by the matrix pipe: with the terms '
-                             'left unformed or five of the six products left out (throw-away builds) they take 65-80 % as long'},
+                             'chain fetch -> LDS -> matrix instructions of a 16-deep chunk, which the two blocks of a compute unit '
+                             'run in step: in throw-away builds the kernel without any matrix instruction still takes 55 % as long, '
+                             'and the parts add up'},
         'wgrad_tflops': round(flops_per_pass * args.steps / (x3_prof['conv_wgrad'][1] * 1e-3) / 1e12, 2),
         'kernels_ms_per_step': {k: round(v[1] / args.steps, 4) for k, v in x3_prof.items() if v[0]}}
     del layers
