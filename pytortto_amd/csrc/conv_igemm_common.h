@@ -80,6 +80,16 @@ struct Igemm {
 };
 
 
+// Several data-parallel launches in one grid (the stride-parity classes of a strided input
+// gradient): blocks [first[i], first[i+1]) belong to launch i.  One grid instead of a short
+// launch per class, each with its own ramp-up and tail.
+constexpr int kMaxMulti = 4;
+struct IgemmMulti {
+  Igemm c[kMaxMulti];
+  int first[kMaxMulti + 1];
+  int n;
+};
+
 constexpr int kModeCompare = 0, kModeGemm = 1, kModeTapMask = 2, kModeTapMask64 = 3;
 constexpr int kSrdFlags = 0x00020000;        // raw buffer, 32-bit data format
 constexpr int kSrdRecords = 0x7fffffff;      // offsets with bit 31 set are out of range and read 0
@@ -90,5 +100,16 @@ __device__ __forceinline__ float as_float(unsigned v) { return __builtin_bit_cas
 // (tile rows `bm` as planned by the caller); `launch` enqueues it on the library stream.
 bool bf16_first_supported(const Igemm& p, int groups, int bm);
 void bf16_first_launch(const Igemm& p, int groups, int bm, hipStream_t st);
+
+
+// Float32 arithmetic in three bf16 terms (conv_igemm_x3.hip: the kernel body of conv_igemm_kernel.h
+// instantiated on six v_mfma_f32_32x32x16_bf16 per product step).  `bm` x `bn` is the tile the caller
+// planned; `sk_blocks` > 0 asks for the persistent (stream-K) grid, which is launched only if the
+// device holds that many blocks at once (`forced_occupancy` >= 0 replaces what the device says:
+// tests); returns whether the persistent grid was launched.
+bool x3_launch(const Igemm& p, int groups, int sk_blocks, int bm, int bn, int forced_occupancy, hipStream_t st);
+void x3_launch_multi(const IgemmMulti& m, int groups, int bm, int bn, hipStream_t st);
+// resident blocks per compute unit of its stream-K kernels, the smallest over every instantiation
+int x3_min_resident_blocks();
 
 }  // namespace ttc
